@@ -1,0 +1,134 @@
+/*
+ * samfast - C ABI of the MI355X (gfx950) SAM image-encoder hot path.
+ *
+ * Two groups of entry points:
+ *   attention with decomposed relative-position bias (global 64-wide grids and
+ *   small windows), and dynamic symmetric int8 linears (row quantiser, int8
+ *   GEMM with int32 accumulators, fused scale+bias epilogue).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless named host_*; the caller owns
+ *     all buffers, nothing is retained after the call returns;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); calls
+ *     only enqueue work, they never synchronise and never allocate;
+ *   - strides are in ELEMENTS; the innermost (head_dim / K) axis is contiguous
+ *     and every row start must be 16-byte aligned;
+ *   - return value 0 = ok; negative = SAMFAST_E_*; the text of the last error
+ *     on the calling thread is returned by samfast_last_error().
+ *
+ * The reference interfaces each entry point stands in for are cited as
+ * file:line under segment_anything_fast/ of pytorch-labs/segment-anything-fast.
+ */
+#ifndef SAMFAST_H
+#define SAMFAST_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SAMFAST_VERSION 1
+
+/* element types of attention operands / linear outputs */
+#define SAMFAST_BF16 0
+#define SAMFAST_F16 1
+
+#define SAMFAST_OK 0
+#define SAMFAST_E_INVALID (-1)      /* bad shape / stride / alignment / null pointer */
+#define SAMFAST_E_UNSUPPORTED (-2)  /* a shape or type no kernel here covers */
+#define SAMFAST_E_LAUNCH (-3)       /* the HIP runtime refused the launch */
+
+int samfast_version(void);
+/* "gfx950" - the only architecture the code objects are built for */
+const char* samfast_arch(void);
+const char* samfast_last_error(void);
+
+/*
+ * out = softmax(q k^T * sm_scale + rel_h[.., kh] + rel_w[.., kw]) v, the bias
+ * computed inside the kernel from the two relative-position tables:
+ *   rel_h[b,h,(y,x),j] = <q[b,h,(y,x),:], rel_pos_h[y - j + gh - 1, :]>
+ *   rel_w[b,h,(y,x),j] = <q[b,h,(y,x),:], rel_pos_w[x - j + gw - 1, :]>
+ * Replaces, in one launch: add_decomposed_rel_pos (modeling/image_encoder.py:338-372,
+ * called at :234) + _attention_rel_h_rel_w (flash_4.py:335-370, called at
+ * modeling/image_encoder.py:245), for both the global (gh=gw=64) and the windowed
+ * (gh=gw=14) blocks.
+ *
+ * q,k,v,out: logical shape (B, nH, N=gh*gw, hd), addressed as
+ *   ptr + b*s_b + h*s_h + n*s_n + d, so head-major (B,nH,N,hd) tensors and the
+ *   token-major output of the qkv Linear ((B,N,3,nH,hd)) are both accepted
+ *   without a copy.
+ * rel_pos_h: (2*gh-1, hd) contiguous, rel_pos_w: (2*gw-1, hd) contiguous, same
+ *   element type as q.
+ * Supported: hd in {64, 80}; (gw == 64 and N % 128 == 0) or (gh <= 15 and
+ *   gw <= 16 and N <= 208); dtype SAMFAST_BF16.
+ */
+int samfast_attn_relpos_fwd(
+    const void* q, const void* k, const void* v,
+    const void* rel_pos_h, const void* rel_pos_w, void* out,
+    int B, int nH, int gh, int gw, int hd,
+    int64_t q_sb, int64_t q_sh, int64_t q_sn,
+    int64_t k_sb, int64_t k_sh, int64_t k_sn,
+    int64_t v_sb, int64_t v_sh, int64_t v_sn,
+    int64_t o_sb, int64_t o_sh, int64_t o_sn,
+    int dtype, float sm_scale, void* stream);
+
+/*
+ * Same attention with the two bias factors already computed by the caller:
+ *   rel_h: (B, nH, N, gh) addressed ptr + b*rh_sb + h*rh_sh + n*rh_sn + j
+ *   rel_w: (B, nH, N, gw) addressed ptr + b*rw_sb + h*rw_sh + n*rw_sn + j
+ * This is the operand form of _attention_rel_h_rel_w(q,k,v,rel_h,rel_w)
+ * (flash_4.py:335) and, with rel_h = base, rel_w = base + 64 and row stride 128,
+ * of the operator customflash::custom_flash_aligned(q,k,v,rel_h_w,sm_scale)
+ * (flash_4.py:268-329).  Same supported shapes as samfast_attn_relpos_fwd.
+ */
+int samfast_attn_relpos_bias_fwd(
+    const void* q, const void* k, const void* v,
+    const void* rel_h, const void* rel_w, void* out,
+    int B, int nH, int gh, int gw, int hd,
+    int64_t q_sb, int64_t q_sh, int64_t q_sn,
+    int64_t k_sb, int64_t k_sh, int64_t k_sn,
+    int64_t v_sb, int64_t v_sh, int64_t v_sn,
+    int64_t o_sb, int64_t o_sh, int64_t o_sn,
+    int64_t rh_sb, int64_t rh_sh, int64_t rh_sn,
+    int64_t rw_sb, int64_t rw_sh, int64_t rw_sn,
+    int dtype, float sm_scale, void* stream);
+
+/*
+ * Per-row symmetric int8 quantiser: for each of M rows of x (K values, row
+ * stride ldx elements, type `dtype`):
+ *   s = max(absmax(row), 1e-5) / 127;  xq = clamp(rint(row / s), -127, 127)
+ * Writes xq (M, K) int8 contiguous and sx (M) fp32.  Stands for the per-token
+ * activation quantiser torchao.apply_dynamic_quant installs in front of every
+ * Linear (call site experiments/eval_combo.py:357-359).  K % 8 == 0, K <= 8192.
+ */
+int samfast_quant_rowwise_i8(
+    const void* x, int64_t ldx, int8_t* xq, float* sx,
+    int64_t M, int K, int dtype, void* stream);
+
+/*
+ * acc[m, n] = sum_k xq[m, k] * wq[n, k], int32, exact.  xq (M, K) and wq (N, K)
+ * int8 contiguous; acc (M, N) int32 contiguous.  The torch._int_mm step of the
+ * quantised Linear (same call site), exposed so accumulators can be compared
+ * bit for bit.  K % 64 == 0, N % 8 == 0.
+ */
+int samfast_gemm_i8_i32(
+    const int8_t* xq, const int8_t* wq, int32_t* acc,
+    int64_t M, int N, int K, void* stream);
+
+/*
+ * y[m, n] = (float(acc[m, n]) * sx[m]) * sw[n] + bias[n], rounded to `dtype`
+ * (bf16), acc as in samfast_gemm_i8_i32 but never written to memory.  bias is
+ * fp32 (N) or NULL; y has row stride ldy elements.  The whole quantised
+ * nn.Linear.forward for qkv / proj (modeling/image_encoder.py:228,251) and
+ * lin1 / lin2 (modeling/common.py:26) after samfast_quant_rowwise_i8.
+ */
+int samfast_gemm_i8_scale_bias(
+    const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
+    const float* bias, void* y, int64_t ldy,
+    int64_t M, int N, int K, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SAMFAST_H */

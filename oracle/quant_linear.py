@@ -1,0 +1,124 @@
+"""Oracle: dynamic symmetric int8 linear (CPU, numpy integers + fp32).
+
+TEST INFRASTRUCTURE ONLY (see the package docstring).
+
+What the reference does on this path
+------------------------------------
+experiments/eval_combo.py:357-360 calls `torchao.quantization.apply_dynamic_quant`
+on the image encoder.  torchao is a third-party dependency that setup.py:16
+names without a version, that is not vendored under the reference tree and is
+not installed here.  Its published algorithm (torchao 0.1, quant_primitives:
+`quantize_activation_per_token_absmax`, `dynamically_quantize_per_channel`,
+`quant_int8_per_token_matmul`) is restated below in the form the benchmark
+configuration of this build fixes it:
+
+  activations, per token (row):  s_x[m] = absmax(x[m, :]) / 127
+  weights, per output channel:   s_w[n] = absmax(w[n, :]) / 127
+  q = clamp(round_half_even(value / s), -127, 127) as int8
+  acc[m, n] = sum_k xq[m, k] * wq[n, k]            (int32, exact)
+  y[m, n]   = (float(acc) * s_x[m]) * s_w[n] + bias[n]   -> bf16
+
+All floating-point steps are single fp32 operations in the order written
+(no fused multiply-add), so a GPU kernel can reproduce them bit for bit.
+An all-zero row or channel gets absmax floored at 1e-5 (torchao's eps), which
+only changes rows that quantise to all zeros anyway.
+
+PARITY UNPINNED against torchao itself: the reference holds no test, golden
+vector or fixture for the quantised path, and torchao cannot be imported in
+this environment, so its exact scale/rounding conventions (127 vs 127.5
+divisors, bf16 vs fp32 division) are not checked.  What IS pinned
+(tests/test_oracle_quant.py): the integer GEMM against int64 matmul and
+torch._int_mm (the library routine torchao calls); the quantisers against
+their closed form and invariants (|q| <= 127, the absmax element maps to
++-127, positive rescaling of a row leaves q unchanged, rows are independent,
+dequantisation error <= s/2); the epilogue against float64.
+"""
+
+import numpy as np
+import torch
+
+EPS = np.float32(1e-5)
+QMAX = np.float32(127.0)
+
+
+def _to_f32_numpy(t) -> np.ndarray:
+    if isinstance(t, torch.Tensor):
+        return t.detach().to(torch.float32).cpu().numpy()
+    return np.asarray(t, dtype=np.float32)
+
+
+def quantize_rows_absmax(x):
+    """Per-row symmetric int8: returns (q int8 (M, K), scale fp32 (M,)).
+
+    Stands for torchao's per-token activation quantiser (called from
+    experiments/eval_combo.py:357-359) and, applied to a (N, K) weight, for
+    its per-output-channel weight quantiser.
+    """
+    xf = _to_f32_numpy(x)
+    assert xf.ndim == 2
+    absmax = np.maximum(np.abs(xf).max(axis=1), EPS).astype(np.float32)
+    scale = (absmax / QMAX).astype(np.float32)
+    ratio = (xf / scale[:, None]).astype(np.float32)
+    q = np.clip(np.rint(ratio), -127.0, 127.0).astype(np.int8)  # rint = half to even
+    return q, scale
+
+
+def int8_gemm_i32(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:
+    """acc[m, n] = sum_k xq[m, k] * wq[n, k] as int32 (torch._int_mm semantics).
+
+    |acc| <= K * 127^2 < 2^31 for K <= 133 000, so int32 never wraps here.
+    """
+    assert xq.dtype == np.int8 and wq.dtype == np.int8
+    M, K = xq.shape
+    N = wq.shape[0]
+    if M > 16 and K % 8 == 0 and N % 8 == 0:
+        # torch._int_mm is multi-threaded; exact for integers like any other route.
+        a = torch.from_numpy(np.ascontiguousarray(xq))
+        b = torch.from_numpy(np.ascontiguousarray(wq)).t()
+        return torch._int_mm(a, b).numpy()
+    return (xq.astype(np.int32) @ wq.astype(np.int32).T).astype(np.int32)
+
+
+def int8_gemm_i64(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:
+    """Same product through int64 numpy matmul: the independent check of int8_gemm_i32."""
+    return xq.astype(np.int64) @ wq.astype(np.int64).T
+
+
+def scale_bias_epilogue(acc: np.ndarray, sx: np.ndarray, sw: np.ndarray, bias) -> torch.Tensor:
+    """y = (float(acc) * sx[m]) * sw[n] + bias[n], each step one fp32 op, -> bf16."""
+    t = acc.astype(np.float32)  # int32 -> fp32, round to nearest even
+    t = (t * sx.astype(np.float32)[:, None]).astype(np.float32)
+    t = (t * sw.astype(np.float32)[None, :]).astype(np.float32)
+    if bias is not None:
+        t = (t + _to_f32_numpy(bias)[None, :]).astype(np.float32)
+    return torch.from_numpy(t).to(torch.bfloat16)
+
+
+def dynamic_int8_linear(x: torch.Tensor, weight: torch.Tensor, bias) -> torch.Tensor:
+    """Whole dynamic-quant Linear on (..., K) activations; returns bf16 (..., N)."""
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1])
+    xq, sx = quantize_rows_absmax(x2)
+    wq, sw = quantize_rows_absmax(weight)
+    acc = int8_gemm_i32(xq, wq)
+    y = scale_bias_epilogue(acc, sx, sw, bias)
+    return y.reshape(*lead, weight.shape[0])
+
+
+def prune_2_of_4(weight: torch.Tensor) -> torch.Tensor:
+    """Zero the 2 smallest-magnitude entries of every 4 consecutive along K.
+
+    Follows segment_anything_fast/sparse.py:6-25 (WeightNormSparsifier with
+    sparse_block_shape=(1, 4), zeros_per_block=2, sparsity_level=1.0).  Ties
+    keep the earlier index (the sparsifier leaves tie order unspecified).
+    """
+    w = _to_f32_numpy(weight)
+    N, K = w.shape
+    assert K % 4 == 0
+    blocks = np.abs(w).reshape(N, K // 4, 4)
+    # stable sort descending by magnitude: keep the first two positions
+    order = np.argsort(-blocks, axis=-1, kind="stable")
+    keep = np.zeros_like(blocks, dtype=bool)
+    np.put_along_axis(keep, order[..., :2], True, axis=-1)
+    out = (w.reshape(N, K // 4, 4) * keep).reshape(N, K)
+    return torch.from_numpy(out).to(weight.dtype if isinstance(weight, torch.Tensor) else torch.float32)

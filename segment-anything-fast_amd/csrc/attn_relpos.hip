@@ -1,0 +1,733 @@
+// Attention with decomposed relative-position bias for gfx950 (bf16 MFMA).
+//
+//   out = softmax(q k^T * sm_scale + rel_h[q, kh] + rel_w[q, kw]) v,   key n = kh*gw + kw
+//
+// Both kernels compute the TRANSPOSED score tile S^T = K Q^T with
+// v_mfma_f32_32x32x16_bf16 (A = 32 keys x 16 channels from LDS, B = Q^T held in
+// registers for the whole kernel).  In the MFMA result layout a lane then owns
+// ONE query (column lane%32) and 16 keys per tile (rows 8*(r/4) + 4*(lane/32) +
+// r%4), so the softmax row statistics are per-lane scalars: the row maximum and
+// sum are reduced in registers plus one exchange with lane^32.  The same
+// registers, converted to bf16, are directly the B operand (P^T) of the second
+// product O^T = V^T P^T, whose A operand is read from a transposed copy of V in
+// LDS with two 8-byte reads that follow the key order of the P registers.
+//
+// Everything runs in the base-2 domain with the exact scale folded into the
+// exponent argument: p = exp2(fma(s, c, -m)), c = sm_scale*log2(e), so q is
+// never re-rounded.
+//
+// global kernel (gw == 64): one key tile is exactly one key grid row, so
+//   rel_w is identical for every key tile -> kept in registers as the INITIAL
+//   accumulator of the score MFMA (pre-divided by sm_scale), and rel_h is one
+//   scalar per (query, key tile) -> folded into the running-max bookkeeping.
+//   With FUSED the two factors are produced in the prologue by MFMA from the
+//   (2S-1, hd) tables: rel_h^T = Rh[qh+gh-1-kh] Q^T directly, rel_w through the
+//   full product T = Rw Q^T followed by the per-query diagonal gather
+//   rel_w[q, kw] = T[qw - kw + 63, q] staged through LDS.
+//
+// window kernel (N <= 208, e.g. 14x14): all keys of one (window, head) fit in
+//   LDS; one pass, no online rescaling.  The bias is added BY THE MFMA: the
+//   channel axis is extended by 32 slots, B carries [rel_h[q, 0..15] | rel_w[q,
+//   0..15]] / sm_scale in bf16 and A carries the 0/1 indicators [n/gw == j |
+//   n%gw == j]; slot 15 of the rel_h half is the padding mask (B = -1e30, A = 1
+//   for key rows >= N).
+#include "samfast_internal.hpp"
+
+namespace samfast {
+
+struct AttnArgs {
+  const unsigned short* q;
+  const unsigned short* k;
+  const unsigned short* v;
+  const unsigned short* rh;  // FUSED: rel_pos_h table (2gh-1, hd); else rel_h (B,nH,N,gh)
+  const unsigned short* rw;  // FUSED: rel_pos_w table (2gw-1, hd); else rel_w (B,nH,N,gw)
+  unsigned short* out;
+  int64_t q_sb, q_sh, q_sn;
+  int64_t k_sb, k_sh, k_sn;
+  int64_t v_sb, v_sh, v_sn;
+  int64_t o_sb, o_sh, o_sn;
+  int64_t rh_sb, rh_sh, rh_sn;
+  int64_t rw_sb, rw_sh, rw_sn;
+  int B, nH, gh, gw, N;
+  float c;          // sm_scale * log2(e)
+  float inv_scale;  // 1 / sm_scale
+};
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+SF_DEVICE bf16x8 as_bf16x8(u32x4 w) { return __builtin_bit_cast(bf16x8, w); }
+
+SF_DEVICE bf16x8 load_bf16x8_global(const unsigned short* p) {
+  return as_bf16x8(*reinterpret_cast<const u32x4*>(p));
+}
+
+SF_DEVICE bf16x8 cvt_bf16x8(const f32x16& s, int base) {
+  u32x4 w;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(s[base + 2 * i], s[base + 2 * i + 1]);
+  return as_bf16x8(w);
+}
+
+// all LDS operations this wavefront has issued are complete and ordered
+SF_DEVICE void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// transpose a 4-key x 8-channel block held as 4 x 16 bytes into 8 x (4 keys) 8-byte rows
+SF_DEVICE void transpose_4x8(const u32x4 (&in)[4], u32x2 (&outv)[8]) {
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const unsigned int k0 = in[0][m], k1 = in[1][m], k2 = in[2][m], k3 = in[3][m];
+    outv[2 * m][0] = (k0 & 0xffffu) | (k1 << 16);
+    outv[2 * m][1] = (k2 & 0xffffu) | (k3 << 16);
+    outv[2 * m + 1][0] = (k0 >> 16) | (k1 & 0xffff0000u);
+    outv[2 * m + 1][1] = (k2 >> 16) | (k3 & 0xffff0000u);
+  }
+}
+
+// =============================================================================
+// global kernel: gw == 64, N % (128*QT) == 0
+// =============================================================================
+template <int HD, int QT>
+struct GlobalCfg {
+  static constexpr int KS = HD / 16;          // score k-steps
+  static constexpr int DT = (HD + 31) / 32;   // output channel tiles
+  static constexpr int BM = 128 * QT;         // queries per workgroup
+  static constexpr int KSTR = HD + 8;         // K row stride in LDS (elements)
+  static constexpr int VSTR = 64 + 8;         // V^T row stride in LDS (elements)
+  static constexpr int KBYTES = 64 * KSTR * 2;
+  static constexpr int VBYTES = HD * VSTR * 2;
+  static constexpr int STAGE = KBYTES + VBYTES;
+  static constexpr int RELH_OFF = 2 * STAGE;
+  static constexpr int RELH_BYTES = 64 * BM * 4;
+  static constexpr int LDS_BYTES = RELH_OFF + RELH_BYTES;
+  static constexpr int XSTR = 65;             // gather scratch row stride (floats)
+  static constexpr int X_BYTES = 4 * 32 * XSTR * 4;
+  static constexpr int KCH = 64 * HD / 8;     // 16-byte chunks in a K tile
+  static constexpr int KLOADS = (KCH + 255) / 256;
+  static constexpr int VBLK = 16 * (HD / 8);  // 4x8 blocks in a V tile
+  static_assert(X_BYTES <= 2 * STAGE, "gather scratch must fit in the K/V stages");
+};
+
+template <int HD, int QT, bool FUSED>
+__global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
+  using C = GlobalCfg<HD, QT>;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[C::LDS_BYTES];
+  float* relhT = reinterpret_cast<float*>(lds + C::RELH_OFF);  // [kh][BM]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 31, lh = lane >> 5;
+
+  const unsigned int nqb = a.N / C::BM;
+  const unsigned int total = (unsigned int)(a.B * a.nH) * nqb;
+  const unsigned int pid = xcd_contiguous_id(blockIdx.x, total);
+  if (pid >= total) return;
+  const int bh = pid / nqb, qb = pid % nqb;
+  const int b = bh / a.nH, h = bh % a.nH;
+  const int q_wg = qb * C::BM;            // first query of the workgroup
+  const int q_wave = wave * 32 * QT;      // first query of the wave inside the workgroup
+
+  const unsigned short* kbase = a.k + b * a.k_sb + h * a.k_sh;
+  const unsigned short* vbase = a.v + b * a.v_sb + h * a.v_sh;
+  const unsigned short* qbase = a.q + b * a.q_sb + h * a.q_sh;
+
+  // ---- staging registers for one K/V tile ----------------------------------
+  u32x4 kst[C::KLOADS];
+  u32x4 vst[4];
+  const int v_kg = tid & 15, v_dg = tid >> 4;
+  const bool v_active = tid < C::VBLK;
+  auto stage_load = [&](int kt) {
+    const int n0 = kt * 64;
+#pragma unroll
+    for (int i = 0; i < C::KLOADS; ++i) {
+      const int c = tid + 256 * i;
+      if (c < C::KCH) {
+        const int row = c / (HD / 8), col = c % (HD / 8);
+        kst[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)(n0 + row) * a.k_sn + col * 8);
+      }
+    }
+    if (v_active) {
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk)
+        vst[kk] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)(n0 + 4 * v_kg + kk) * a.v_sn + v_dg * 8);
+    }
+  };
+  auto stage_store = [&](int buf) {
+    unsigned char* kl = lds + buf * C::STAGE;
+    unsigned char* vl = kl + C::KBYTES;
+#pragma unroll
+    for (int i = 0; i < C::KLOADS; ++i) {
+      const int c = tid + 256 * i;
+      if (c < C::KCH) {
+        const int row = c / (HD / 8), col = c % (HD / 8);
+        *reinterpret_cast<u32x4*>(kl + (row * C::KSTR + col * 8) * 2) = kst[i];
+      }
+    }
+    if (v_active) {
+      u32x2 t[8];
+      transpose_4x8(vst, t);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *reinterpret_cast<u32x2*>(vl + ((v_dg * 8 + i) * C::VSTR + 4 * v_kg) * 2) = t[i];
+    }
+  };
+
+  stage_load(0);
+
+  // ---- Q^T operand: lane holds query lr of tile t, channels 16s + 8lh .. +7 ----
+  bf16x8 qf[QT][C::KS];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    const unsigned short* qp = qbase + (int64_t)(q_wg + q_wave + 32 * t + lr) * a.q_sn + 8 * lh;
+#pragma unroll
+    for (int s = 0; s < C::KS; ++s) qf[t][s] = load_bf16x8_global(qp + 16 * s);
+  }
+
+  // ---- bias prologue -----------------------------------------------------------
+  // b1[t][nt][r]: rel_w / sm_scale for the lane's query and key column kw of the
+  // score-tile layout.  relhT[kh][q]: rel_h * log2(e).
+  f32x16 b1[QT][2];
+  if (FUSED) {
+    const unsigned short* th = a.rh;
+    const unsigned short* tw = a.rw;
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+      const int qh = (q_wg + q_wave + 32 * t) >> 6;  // one grid row per 32-query tile
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const int kh_row = 32 * mt + lr;
+        int trow = qh - kh_row + a.gh - 1;
+        trow = max(0, min(trow, 2 * a.gh - 2));
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < C::KS; ++s) {
+          const bf16x8 av = load_bf16x8_global(th + trow * HD + 16 * s + 8 * lh);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[t][s], acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int kh = 32 * mt + 8 * (r >> 2) + 4 * lh + (r & 3);
+          relhT[kh * C::BM + q_wave + 32 * t + lr] = acc[r] * kLog2e;
+        }
+      }
+    }
+    // rel_w: T[rel][q] for rel in [0,128) in two passes of 64 through LDS scratch
+    float* X = reinterpret_cast<float*>(lds) + wave * 32 * C::XSTR;
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+      const int qw = (q_wg + q_wave + 32 * t + lr) & 63;
+#pragma unroll
+      for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int mt = 2 * pass + half;
+          const int trow = min(32 * mt + lr, 126);
+          f32x16 acc;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+          for (int s = 0; s < C::KS; ++s) {
+            const bf16x8 av = load_bf16x8_global(tw + trow * HD + 16 * s + 8 * lh);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[t][s], acc, 0, 0, 0);
+          }
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int rel_local = 32 * half + 8 * (r >> 2) + 4 * lh + (r & 3);
+            X[lr * C::XSTR + rel_local] = acc[r];
+          }
+        }
+        wave_lds_fence();
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int kw = 32 * nt + 8 * (r >> 2) + 4 * lh + (r & 3);
+            const int rel = qw + 63 - kw;
+            const float val = X[lr * C::XSTR + (rel & 63)] * a.inv_scale;  // always in range
+            if (pass == 0) b1[t][nt][r] = val;
+            else b1[t][nt][r] = (rel >= 64) ? val : b1[t][nt][r];
+          }
+        wave_lds_fence();
+      }
+    }
+  } else {
+    const unsigned short* rhb = a.rh + b * a.rh_sb + h * a.rh_sh + (int64_t)q_wg * a.rh_sn;
+    for (int idx = tid; idx < C::BM * a.gh; idx += 256) {
+      const int ql = idx % C::BM, kh = idx / C::BM;
+      relhT[kh * C::BM + ql] = bf16_bits_to_f32(rhb[(int64_t)ql * a.rh_sn + kh]) * kLog2e;
+    }
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+      const unsigned short* rwp =
+          a.rw + b * a.rw_sb + h * a.rw_sh + (int64_t)(q_wg + q_wave + 32 * t + lr) * a.rw_sn;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const u32x2 w = *reinterpret_cast<const u32x2*>(rwp + 32 * nt + 8 * j + 4 * lh);
+          b1[t][nt][4 * j + 0] = bf16_lo_to_f32(w[0]) * a.inv_scale;
+          b1[t][nt][4 * j + 1] = bf16_hi_to_f32(w[0]) * a.inv_scale;
+          b1[t][nt][4 * j + 2] = bf16_lo_to_f32(w[1]) * a.inv_scale;
+          b1[t][nt][4 * j + 3] = bf16_hi_to_f32(w[1]) * a.inv_scale;
+        }
+    }
+  }
+  __syncthreads();  // scratch reads done, relhT complete
+  stage_store(0);
+  __syncthreads();
+
+  // ---- main loop over key grid rows ---------------------------------------------
+  f32x16 oacc[QT][C::DT];
+  float m_i[QT], l_i[QT];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    m_i[t] = -INFINITY;
+    l_i[t] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[t][dt][r] = 0.f;
+  }
+
+  const int nkt = a.N / 64;
+  for (int kt = 0; kt < nkt; ++kt) {
+    const unsigned char* kl = lds + (kt & 1) * C::STAGE;
+    const unsigned char* vl = kl + C::KBYTES;
+    const bool more = kt + 1 < nkt;
+    if (more) stage_load(kt + 1);
+
+    // S^T = K Q^T, accumulator initialised with rel_w / sm_scale
+    f32x16 s[QT][2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+      for (int t = 0; t < QT; ++t) s[t][nt] = b1[t][nt];
+#pragma unroll
+      for (int ks = 0; ks < C::KS; ++ks) {
+        const bf16x8 av = as_bf16x8(*reinterpret_cast<const u32x4*>(
+            kl + ((32 * nt + lr) * C::KSTR + 16 * ks + 8 * lh) * 2));
+#pragma unroll
+        for (int t = 0; t < QT; ++t)
+          s[t][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[t][ks], s[t][nt], 0, 0, 0);
+      }
+    }
+
+    // online softmax, one query per lane
+    bf16x8 pk[QT][4];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+      float mx = s[t][0][0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[t][0][r]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[t][1][r]);
+      mx = fmaxf(mx, xor32(mx));
+      const float b0 = relhT[kt * C::BM + q_wave + 32 * t + lr];
+      const float m_new = fmaxf(m_i[t], fmaf(mx, a.c, b0));
+      const float alpha = fast_exp2(m_i[t] - m_new);
+      m_i[t] = m_new;
+      const float neg_mrow = b0 - m_new;
+      float lsum = 0.f;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float p = fast_exp2(fmaf(s[t][nt][r], a.c, neg_mrow));
+          s[t][nt][r] = p;
+          lsum += p;
+        }
+      l_i[t] = l_i[t] * alpha + lsum;
+      if (__any(alpha != 1.0f)) {
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[t][dt][r] *= alpha;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pk[t][j] = cvt_bf16x8(s[t][j >> 1], 8 * (j & 1));
+    }
+
+    // O^T += V^T P^T
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int dt = 0; dt < C::DT; ++dt) {
+        const int drow = min(32 * dt + lr, HD - 1);
+        const unsigned char* vp = vl + (drow * C::VSTR + 16 * j + 4 * lh) * 2;
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 16);
+        const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+        const bf16x8 av = as_bf16x8(w);
+#pragma unroll
+        for (int t = 0; t < QT; ++t)
+          oacc[t][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, pk[t][j], oacc[t][dt], 0, 0, 0);
+      }
+    }
+
+    if (more) stage_store((kt + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: O = acc / l, 4 adjacent channels per store --------------------
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    const float l = l_i[t] + xor32(l_i[t]);
+    const float inv = 1.0f / l;
+    unsigned short* op = a.out + b * a.o_sb + h * a.o_sh + (int64_t)(q_wg + q_wave + 32 * t + lr) * a.o_sn;
+#pragma unroll
+    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = 32 * dt + 8 * j + 4 * lh;
+        if (d < HD) {
+          const u32x2 o = {pack_bf16x2(oacc[t][dt][4 * j] * inv, oacc[t][dt][4 * j + 1] * inv),
+                           pack_bf16x2(oacc[t][dt][4 * j + 2] * inv, oacc[t][dt][4 * j + 3] * inv)};
+          *reinterpret_cast<u32x2*>(op + d) = o;
+        }
+      }
+  }
+}
+
+// =============================================================================
+// window kernel: gh <= 15, gw <= 16, N = gh*gw <= 208; one workgroup per (b, head)
+// =============================================================================
+template <int HD>
+struct WindowCfg {
+  static constexpr int KS = HD / 16;
+  static constexpr int DT = (HD + 31) / 32;
+  static constexpr int NMAX = 208;
+  static constexpr int NT = 7;                 // score tiles of 32 keys
+  static constexpr int KSTR = HD + 8;
+  static constexpr int VSTR = NMAX + 4;
+  static constexpr int KBYTES = NMAX * KSTR * 2;
+  static constexpr int VBYTES = HD * VSTR * 2;
+  static constexpr int XSTR = 34;              // bf16 elements per scratch row
+  static constexpr int XBYTES_WAVE = 32 * XSTR * 2;      // one bias factor at a time
+  static constexpr int X_OFF = KBYTES + VBYTES;
+  static constexpr int LDS_BYTES = X_OFF + 4 * XBYTES_WAVE;
+};
+
+// one-hot bf16x8: element e is 1.0 iff slot == 8*lh + e
+SF_DEVICE bf16x8 onehot_bf16x8(int slot, int lh) {
+  const int e = slot - 8 * lh;  // may be outside [0, 8)
+  u32x4 w;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    unsigned int v = 0u;
+    if ((e >> 1) == i) v = (e & 1) ? 0x3F800000u : 0x00003F80u;
+    w[i] = v;
+  }
+  return as_bf16x8(w);
+}
+
+template <int HD, bool FUSED>
+__global__ __launch_bounds__(256, 2) void attn_window_kernel(AttnArgs a) {
+  using C = WindowCfg<HD>;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[C::LDS_BYTES];
+  unsigned char* kl = lds;
+  unsigned char* vl = lds + C::KBYTES;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 31, lh = lane >> 5;
+  const int N = a.N;
+  const int bh = blockIdx.x;
+  const int b = bh / a.nH, h = bh % a.nH;
+
+  const unsigned short* kbase = a.k + b * a.k_sb + h * a.k_sh;
+  const unsigned short* vbase = a.v + b * a.v_sb + h * a.v_sh;
+  const unsigned short* qbase = a.q + b * a.q_sb + h * a.q_sh;
+
+  // ---- K rows -> LDS; V 4x8 blocks -> transposed LDS (zero beyond N) -----------
+  {
+    const int nch = N * (HD / 8);
+    for (int c = tid; c < nch; c += 256) {
+      const int row = c / (HD / 8), col = c % (HD / 8);
+      const u32x4 w = *reinterpret_cast<const u32x4*>(kbase + (int64_t)row * a.k_sn + col * 8);
+      *reinterpret_cast<u32x4*>(kl + (row * C::KSTR + col * 8) * 2) = w;
+    }
+    const int nkg = 4 * ((N + 15) / 16);  // key groups of 4, up to the 16-key step boundary
+    const int nblk = nkg * (HD / 8);
+    for (int blk = tid; blk < nblk; blk += 256) {
+      const int kg = blk % nkg, dg = blk / nkg;
+      u32x4 in[4];
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const int key = 4 * kg + kk;
+        u32x4 w = {0u, 0u, 0u, 0u};
+        if (key < N) w = *reinterpret_cast<const u32x4*>(vbase + (int64_t)key * a.v_sn + dg * 8);
+        in[kk] = w;
+      }
+      u32x2 t[8];
+      transpose_4x8(in, t);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *reinterpret_cast<u32x2*>(vl + ((dg * 8 + i) * C::VSTR + 4 * kg) * 2) = t[i];
+    }
+  }
+  __syncthreads();
+
+  const int ntq = (N + 31) / 32;
+  const int nsteps = (N + 15) / 16;
+  unsigned short* X = reinterpret_cast<unsigned short*>(lds + C::X_OFF + wave * C::XBYTES_WAVE);
+
+  for (int t = wave; t < ntq; t += 4) {  // wave-uniform
+    const int qi = 32 * t + lr;
+    const bool q_valid = qi < N;
+    const int qc = min(qi, N - 1);
+    const int qh = qc / a.gw, qw = qc - qh * a.gw;
+
+    bf16x8 qf[C::KS];
+    {
+      const unsigned short* qp = qbase + (int64_t)qc * a.q_sn + 8 * lh;
+#pragma unroll
+      for (int s = 0; s < C::KS; ++s) qf[s] = load_bf16x8_global(qp + 16 * s);
+    }
+
+    // ---- bias operands: lane (query, lh) element e <-> slot 8*lh + e -----------
+    unsigned int bhw[4], bww[4];
+    if (FUSED) {
+      // Th[rel][q], Tw[rel][q] for rel in [0,32): one MFMA row tile each, staged
+      // one after the other through the wave's scratch rows
+      f32x16 th, tw;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { th[r] = 0.f; tw[r] = 0.f; }
+      const int rowh = min(lr, 2 * a.gh - 2), roww = min(lr, 2 * a.gw - 2);
+#pragma unroll
+      for (int s = 0; s < C::KS; ++s) {
+        const bf16x8 ah = load_bf16x8_global(a.rh + rowh * HD + 16 * s + 8 * lh);
+        const bf16x8 aw = load_bf16x8_global(a.rw + roww * HD + 16 * s + 8 * lh);
+        th = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, qf[s], th, 0, 0, 0);
+        tw = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aw, qf[s], tw, 0, 0, 0);
+      }
+#pragma unroll
+      for (int which = 0; which < 2; ++which) {
+        const int g = which ? a.gw : a.gh;
+        const int qpos = which ? qw : qh;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int rel = 8 * (r >> 2) + 4 * lh + (r & 3);
+          const float val = (which ? tw[r] : th[r]) * a.inv_scale;
+          X[lr * C::XSTR + rel] = (unsigned short)f32_to_bf16_bits(val);
+        }
+        wave_lds_fence();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          unsigned int pk2 = 0u;
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int slot = 8 * lh + 2 * i + u;
+            // unconditional read at a clamped position, then select
+            const unsigned int raw = X[lr * C::XSTR + max(0, min(qpos - slot + g - 1, 31))];
+            pk2 |= ((slot < g) ? raw : 0u) << (16 * u);
+          }
+          if (which) bww[i] = pk2; else bhw[i] = pk2;
+        }
+        wave_lds_fence();
+      }
+    } else {
+      const unsigned short* rhp = a.rh + b * a.rh_sb + h * a.rh_sh + (int64_t)qc * a.rh_sn;
+      const unsigned short* rwp = a.rw + b * a.rw_sb + h * a.rw_sh + (int64_t)qc * a.rw_sn;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float fh[2] = {0.f, 0.f}, fw[2] = {0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int slot = 8 * lh + 2 * i + u;
+          const float rh_raw = bf16_bits_to_f32(rhp[min(slot, a.gh - 1)]) * a.inv_scale;
+          const float rw_raw = bf16_bits_to_f32(rwp[min(slot, a.gw - 1)]) * a.inv_scale;
+          fh[u] = (slot < a.gh) ? rh_raw : 0.f;
+          fw[u] = (slot < a.gw) ? rw_raw : 0.f;
+        }
+        bhw[i] = pack_bf16x2(fh[0], fh[1]);
+        bww[i] = pack_bf16x2(fw[0], fw[1]);
+      }
+    }
+    if (lh == 1) bhw[3] = (bhw[3] & 0xffffu) | 0xF1490000u;  // slot 15 = -1e30 (bf16 0xF149)
+    const u32x4 bhv = {bhw[0], bhw[1], bhw[2], bhw[3]};
+    const u32x4 bwv = {bww[0], bww[1], bww[2], bww[3]};
+    const bf16x8 bh_op = as_bf16x8(bhv), bw_op = as_bf16x8(bwv);
+
+    // ---- S^T tiles --------------------------------------------------------------
+    f32x16 s[C::NT];
+    float mx = -3.0e38f;
+#pragma unroll
+    for (int nt = 0; nt < C::NT; ++nt) {
+      if (32 * nt < N) {  // uniform
+        const int n = 32 * nt + lr;
+        const int nc = min(n, N - 1);
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < C::KS; ++ks) {
+          const bf16x8 av = as_bf16x8(
+              *reinterpret_cast<const u32x4*>(kl + (nc * C::KSTR + 16 * ks + 8 * lh) * 2));
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[ks], acc, 0, 0, 0);
+        }
+        const int nh = n / a.gw;
+        const bf16x8 ih = onehot_bf16x8(n < N ? nh : 15, lh);
+        const bf16x8 iw = onehot_bf16x8(n < N ? n - nh * a.gw : 99, lh);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ih, bh_op, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(iw, bw_op, acc, 0, 0, 0);
+        s[nt] = acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, acc[r]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[nt][r] = -1.0e30f;
+      }
+    }
+    mx = fmaxf(mx, xor32(mx));
+    const float neg_m = -mx * a.c;
+
+    // ---- P and O^T = V^T P^T, one score tile (two 16-key steps) at a time -----
+    f32x16 oacc[C::DT];
+#pragma unroll
+    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+    float lsum = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < C::NT; ++nt) {
+      if (2 * nt < nsteps) {  // uniform
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float p = fast_exp2(fmaf(s[nt][r], a.c, neg_m));
+          s[nt][r] = p;
+          lsum += p;
+        }
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int j = 2 * nt + half;
+          if (j < nsteps) {  // uniform
+            const bf16x8 pk = cvt_bf16x8(s[nt], 8 * half);
+#pragma unroll
+            for (int dt = 0; dt < C::DT; ++dt) {
+              const int drow = min(32 * dt + lr, HD - 1);
+              const unsigned char* vp = vl + (drow * C::VSTR + 16 * j + 4 * lh) * 2;
+              const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
+              const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 16);
+              const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+              oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(w), pk, oacc[dt], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+    const float l = lsum + xor32(lsum);
+    const float inv = 1.0f / l;
+    if (q_valid) {
+      unsigned short* op = a.out + b * a.o_sb + h * a.o_sh + (int64_t)qi * a.o_sn;
+#pragma unroll
+      for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int d = 32 * dt + 8 * j + 4 * lh;
+          if (d < HD) {
+            const u32x2 o = {pack_bf16x2(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
+                             pack_bf16x2(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
+            *reinterpret_cast<u32x2*>(op + d) = o;
+          }
+        }
+    }
+  }
+}
+
+// =============================================================================
+// host side
+// =============================================================================
+template <int HD, bool FUSED>
+static int launch_hd(const AttnArgs& a, bool global_path, hipStream_t stream) {
+  if (global_path) {
+    constexpr int QT = 1;
+    using C = GlobalCfg<HD, QT>;
+    const int64_t total = (int64_t)a.B * a.nH * (a.N / C::BM);
+    const unsigned int grid = (unsigned int)(((total + 7) / 8) * 8);
+    hipLaunchKernelGGL((attn_global_kernel<HD, QT, FUSED>), dim3(grid), dim3(256), 0, stream, a);
+    return check_launch("attn_global_kernel");
+  }
+  const unsigned int grid = (unsigned int)(a.B * a.nH);
+  hipLaunchKernelGGL((attn_window_kernel<HD, FUSED>), dim3(grid), dim3(256), 0, stream, a);
+  return check_launch("attn_window_kernel");
+}
+
+static int attn_dispatch(bool fused, AttnArgs& a, int hd, int dtype, float sm_scale,
+                         hipStream_t stream) {
+  SF_REQUIRE(a.q && a.k && a.v && a.out && a.rh && a.rw, "attn_relpos: null pointer");
+  SF_REQUIRE(a.B > 0 && a.nH > 0 && a.gh > 0 && a.gw > 0, "attn_relpos: bad shape");
+  SF_REQUIRE(sm_scale > 0.f, "attn_relpos: sm_scale must be positive");
+  if (dtype != SAMFAST_BF16) SF_FAIL(SAMFAST_E_UNSUPPORTED, "attn_relpos: only bf16 is built");
+  if (hd != 64 && hd != 80)
+    SF_FAIL(SAMFAST_E_UNSUPPORTED, "attn_relpos: head_dim %d not in {64, 80}", hd);
+  SF_REQUIRE((int64_t)a.B * a.nH < (1ll << 24), "attn_relpos: B*nH too large");
+  a.N = a.gh * a.gw;
+  const bool global_path = (a.gw == 64) && (a.N % 128 == 0) && (a.gh <= 64);
+  const bool window_path = (a.gh <= 15) && (a.gw <= 16) && (a.N <= 208);
+  if (!global_path && !window_path)
+    SF_FAIL(SAMFAST_E_UNSUPPORTED,
+            "attn_relpos: grid %dx%d is neither 64-wide (rows even, <= 64) nor a window of <= 15x16",
+            a.gh, a.gw);
+  // every row start 16-byte aligned: strides multiples of 8 elements
+  const int64_t st[12] = {a.q_sb, a.q_sh, a.q_sn, a.k_sb, a.k_sh, a.k_sn,
+                          a.v_sb, a.v_sh, a.v_sn, a.o_sb, a.o_sh, a.o_sn};
+  for (int i = 0; i < 12; ++i)
+    SF_REQUIRE(st[i] >= 0 && st[i] % 8 == 0, "attn_relpos: stride %d = %lld is not a multiple of 8",
+               i, (long long)st[i]);
+  SF_REQUIRE(aligned16(a.q) && aligned16(a.k) && aligned16(a.v) && aligned16(a.out),
+             "attn_relpos: q/k/v/out must be 16-byte aligned");
+  SF_REQUIRE(a.q_sn >= hd && a.k_sn >= hd && a.v_sn >= hd && a.o_sn >= hd,
+             "attn_relpos: token stride smaller than head_dim");
+  if (fused) {
+    SF_REQUIRE(aligned16(a.rh) && aligned16(a.rw), "attn_relpos: tables must be 16-byte aligned");
+  } else if (global_path) {
+    SF_REQUIRE((reinterpret_cast<uintptr_t>(a.rw) & 7u) == 0 && a.rw_sb % 4 == 0 &&
+                   a.rw_sh % 4 == 0 && a.rw_sn % 4 == 0,
+               "attn_relpos: rel_w rows must be 8-byte aligned");
+  }
+  a.c = sm_scale * kLog2e;
+  a.inv_scale = 1.0f / sm_scale;
+  if (hd == 64)
+    return fused ? launch_hd<64, true>(a, global_path, stream) : launch_hd<64, false>(a, global_path, stream);
+  return fused ? launch_hd<80, true>(a, global_path, stream) : launch_hd<80, false>(a, global_path, stream);
+}
+
+}  // namespace samfast
+
+extern "C" int samfast_attn_relpos_fwd(
+    const void* q, const void* k, const void* v, const void* rel_pos_h, const void* rel_pos_w,
+    void* out, int B, int nH, int gh, int gw, int hd,
+    int64_t q_sb, int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+    int64_t v_sb, int64_t v_sh, int64_t v_sn, int64_t o_sb, int64_t o_sh, int64_t o_sn,
+    int dtype, float sm_scale, void* stream) {
+  using us = unsigned short;
+  samfast::AttnArgs a = {};
+  a.q = (const us*)q; a.k = (const us*)k; a.v = (const us*)v;
+  a.rh = (const us*)rel_pos_h; a.rw = (const us*)rel_pos_w; a.out = (us*)out;
+  a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
+  a.B = B; a.nH = nH; a.gh = gh; a.gw = gw;
+  return samfast::attn_dispatch(true, a, hd, dtype, sm_scale, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int samfast_attn_relpos_bias_fwd(
+    const void* q, const void* k, const void* v, const void* rel_h, const void* rel_w, void* out,
+    int B, int nH, int gh, int gw, int hd,
+    int64_t q_sb, int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+    int64_t v_sb, int64_t v_sh, int64_t v_sn, int64_t o_sb, int64_t o_sh, int64_t o_sn,
+    int64_t rh_sb, int64_t rh_sh, int64_t rh_sn, int64_t rw_sb, int64_t rw_sh, int64_t rw_sn,
+    int dtype, float sm_scale, void* stream) {
+  using us = unsigned short;
+  samfast::AttnArgs a = {};
+  a.q = (const us*)q; a.k = (const us*)k; a.v = (const us*)v;
+  a.rh = (const us*)rel_h; a.rw = (const us*)rel_w; a.out = (us*)out;
+  a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
+  a.rh_sb = rh_sb; a.rh_sh = rh_sh; a.rh_sn = rh_sn;
+  a.rw_sb = rw_sb; a.rw_sh = rw_sh; a.rw_sn = rw_sn;
+  a.B = B; a.nH = nH; a.gh = gh; a.gw = gw;
+  SF_REQUIRE(rh_sb >= 0 && rh_sh >= 0 && rh_sn >= 0 && rw_sb >= 0 && rw_sh >= 0 && rw_sn >= 0,
+             "attn_relpos_bias: negative bias stride");
+  return samfast::attn_dispatch(false, a, hd, dtype, sm_scale, reinterpret_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,71 @@
+// Shared device/host helpers of the samfast HIP kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "samfast.h"
+
+namespace samfast {
+
+// ---- error reporting (host) -------------------------------------------------
+void set_error(const char* fmt, ...);
+#define SF_FAIL(code, ...)              \
+  do {                                  \
+    ::samfast::set_error(__VA_ARGS__);  \
+    return (code);                      \
+  } while (0)
+#define SF_REQUIRE(cond, ...)                              \
+  do {                                                     \
+    if (!(cond)) SF_FAIL(SAMFAST_E_INVALID, __VA_ARGS__);  \
+  } while (0)
+
+int check_launch(const char* what);
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- vector types -------------------------------------------------------------
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+#define SF_DEVICE __device__ __forceinline__
+
+// bf16 <-> fp32 on raw bits
+SF_DEVICE float bf16_lo_to_f32(unsigned int w) { return __uint_as_float(w << 16); }
+SF_DEVICE float bf16_hi_to_f32(unsigned int w) { return __uint_as_float(w & 0xffff0000u); }
+SF_DEVICE float bf16_bits_to_f32(unsigned short h) { return __uint_as_float(((unsigned int)h) << 16); }
+
+// round-to-nearest-even fp32 -> bf16 bits (finite inputs; NaN kept quiet)
+SF_DEVICE unsigned int f32_to_bf16_bits(float f) {
+  unsigned int u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+SF_DEVICE unsigned int pack_bf16x2(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+SF_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// value held by lane (lane ^ 32) of the same wavefront
+SF_DEVICE float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+// Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its
+// own L2.  Map the hardware id to a logical id so that every XCD walks one
+// contiguous range of logical ids (neighbours then share an L2).
+SF_DEVICE unsigned int xcd_contiguous_id(unsigned int hw_id, unsigned int total) {
+  const unsigned int per = (total + 7u) >> 3;
+  return (hw_id & 7u) * per + (hw_id >> 3);
+}
+
+}  // namespace samfast

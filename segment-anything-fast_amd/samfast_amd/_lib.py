@@ -1,0 +1,62 @@
+"""ctypes binding of libsamfast.so (the C ABI declared in include/samfast.h).
+
+The library is looked up next to this package (lib/libsamfast.so, built in-tree
+by segment-anything-fast_amd/build.py).  There is no fallback: if it is missing
+or a call fails, a RuntimeError carrying samfast_last_error() is raised.
+"""
+
+import ctypes
+import os
+from pathlib import Path
+
+_LIB_PATH = Path(__file__).resolve().parent / "lib" / "libsamfast.so"
+_lib = None
+
+SAMFAST_BF16 = 0
+SAMFAST_F16 = 1
+
+_i32, _i64, _f32, _ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+
+_SIGNATURES = {
+    "samfast_version": (_i32, []),
+    "samfast_arch": (ctypes.c_char_p, []),
+    "samfast_last_error": (ctypes.c_char_p, []),
+    "samfast_attn_relpos_fwd": (
+        _i32, [_ptr] * 6 + [_i32] * 5 + [_i64] * 12 + [_i32, _f32, _ptr]),
+    "samfast_attn_relpos_bias_fwd": (
+        _i32, [_ptr] * 6 + [_i32] * 5 + [_i64] * 18 + [_i32, _f32, _ptr]),
+    "samfast_quant_rowwise_i8": (_i32, [_ptr, _i64, _ptr, _ptr, _i64, _i32, _i32, _ptr]),
+    "samfast_gemm_i8_i32": (_i32, [_ptr, _ptr, _ptr, _i64, _i32, _i32, _ptr]),
+    "samfast_gemm_i8_scale_bias": (
+        _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _ptr]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def lib_path() -> Path:
+    return Path(os.environ.get("SAMFAST_LIB", str(_LIB_PATH)))
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        path = lib_path()
+        if not path.exists():
+            raise RuntimeError(
+                f"samfast: {path} not found - build it with "
+                "`python segment-anything-fast_amd/build.py` (there is no fallback path)")
+        lib = ctypes.CDLL(str(path))
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+    return _lib
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = load().samfast_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"samfast: {what} failed ({code}): {msg}")

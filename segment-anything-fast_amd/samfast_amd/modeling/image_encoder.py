@@ -1,0 +1,257 @@
+"""SAM ViT image encoder with the hot path on the HIP kernels.
+
+Class names, constructor signatures, parameter names (hence state-dict keys) and
+tensor contracts follow segment_anything_fast/modeling/image_encoder.py:
+ImageEncoderViT :18-117, Block :120-183, Attention :186-253, window_partition
+:256-277, window_unpartition :280-302, get_rel_pos :305-335,
+add_decomposed_rel_pos :338-372, PatchEmbed :375-406.
+
+What differs is Attention.forward on a GPU in bf16: q, k and v are read by the
+attention kernel straight out of the qkv Linear's (B, N, 3, nH, hd) output
+through strides, the two bias factors are computed inside the kernel from
+rel_pos_h / rel_pos_w, and the result is written token-major, so the head
+split/merge copies (:228-230, :249) and the bias tensors (:234-242) never exist.
+Any other input (CPU, fp32, shapes the kernels do not cover) follows the
+reference's own composition through flash_4._attention_rel_h_rel_w.
+"""
+
+from typing import Optional, Tuple, Type
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .. import ops
+from ..flash_4 import USE_CUSTOM_KERNEL, _attention_rel_h_rel_w
+from .common import LayerNorm2d, MLPBlock
+
+
+class ImageEncoderViT(nn.Module):
+    def __init__(
+        self,
+        img_size: int = 1024,
+        patch_size: int = 16,
+        in_chans: int = 3,
+        embed_dim: int = 768,
+        depth: int = 12,
+        num_heads: int = 12,
+        mlp_ratio: float = 4.0,
+        out_chans: int = 256,
+        qkv_bias: bool = True,
+        norm_layer: Type[nn.Module] = nn.LayerNorm,
+        act_layer: Type[nn.Module] = nn.GELU,
+        use_abs_pos: bool = True,
+        use_rel_pos: bool = False,
+        rel_pos_zero_init: bool = True,
+        window_size: int = 0,
+        global_attn_indexes: Tuple[int, ...] = (),
+    ) -> None:
+        super().__init__()
+        self.img_size = img_size
+        grid = img_size // patch_size
+        self.patch_embed = PatchEmbed(
+            kernel_size=(patch_size, patch_size), stride=(patch_size, patch_size),
+            in_chans=in_chans, embed_dim=embed_dim)
+        self.pos_embed: Optional[nn.Parameter] = None
+        if use_abs_pos:
+            self.pos_embed = nn.Parameter(torch.zeros(1, grid, grid, embed_dim))
+        self.blocks = nn.ModuleList([
+            Block(
+                dim=embed_dim, num_heads=num_heads, mlp_ratio=mlp_ratio, qkv_bias=qkv_bias,
+                norm_layer=norm_layer, act_layer=act_layer, use_rel_pos=use_rel_pos,
+                rel_pos_zero_init=rel_pos_zero_init,
+                window_size=0 if i in global_attn_indexes else window_size,
+                input_size=(grid, grid))
+            for i in range(depth)
+        ])
+        self.neck = nn.Sequential(
+            nn.Conv2d(embed_dim, out_chans, kernel_size=1, bias=False),
+            LayerNorm2d(out_chans),
+            nn.Conv2d(out_chans, out_chans, kernel_size=3, padding=1, bias=False),
+            LayerNorm2d(out_chans),
+        )
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        x = self.patch_embed(x)
+        if self.pos_embed is not None:
+            x = x + self.pos_embed
+        for blk in self.blocks:
+            x = blk(x)
+        return self.neck(x.permute(0, 3, 1, 2))
+
+
+class Block(nn.Module):
+    """Pre-norm transformer block; window_size > 0 runs attention inside
+    non-overlapping windows, 0 runs it over the whole grid."""
+
+    def __init__(
+        self,
+        dim: int,
+        num_heads: int,
+        mlp_ratio: float = 4.0,
+        qkv_bias: bool = True,
+        norm_layer: Type[nn.Module] = nn.LayerNorm,
+        act_layer: Type[nn.Module] = nn.GELU,
+        use_rel_pos: bool = False,
+        rel_pos_zero_init: bool = True,
+        window_size: int = 0,
+        input_size: Optional[Tuple[int, int]] = None,
+    ) -> None:
+        super().__init__()
+        self.norm1 = norm_layer(dim)
+        self.attn = Attention(
+            dim, num_heads=num_heads, qkv_bias=qkv_bias, use_rel_pos=use_rel_pos,
+            rel_pos_zero_init=rel_pos_zero_init,
+            input_size=input_size if window_size == 0 else (window_size, window_size))
+        self.norm2 = norm_layer(dim)
+        self.mlp = MLPBlock(embedding_dim=dim, mlp_dim=int(dim * mlp_ratio), act=act_layer)
+        self.window_size = window_size
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        shortcut = x
+        x = self.norm1(x)
+        if self.window_size > 0:
+            H, W = x.shape[1], x.shape[2]
+            x, pad_hw = window_partition(x, self.window_size)
+        x = self.attn(x)
+        if self.window_size > 0:
+            x = window_unpartition(x, self.window_size, pad_hw, (H, W))
+        x = shortcut + x
+        return x + self.mlp(self.norm2(x))
+
+
+class Attention(nn.Module):
+    """Multi-head attention over a (B, H, W, C) token grid with decomposed
+    relative-position bias."""
+
+    def __init__(
+        self,
+        dim: int,
+        num_heads: int = 8,
+        qkv_bias: bool = True,
+        use_rel_pos: bool = False,
+        rel_pos_zero_init: bool = True,
+        input_size: Optional[Tuple[int, int]] = None,
+    ) -> None:
+        super().__init__()
+        self.num_heads = num_heads
+        head_dim = dim // num_heads
+        self.scale = head_dim ** -0.5
+        self.qkv = nn.Linear(dim, dim * 3, bias=qkv_bias)
+        self.proj = nn.Linear(dim, dim)
+        self.use_rel_pos = use_rel_pos
+        if self.use_rel_pos:
+            assert input_size is not None, \
+                "Input size must be provided if using relative positional encoding."
+            self.rel_pos_h = nn.Parameter(torch.zeros(2 * input_size[0] - 1, head_dim))
+            self.rel_pos_w = nn.Parameter(torch.zeros(2 * input_size[1] - 1, head_dim))
+
+    def _fused_ok(self, qkv: torch.Tensor, H: int, W: int, hd: int) -> bool:
+        return (self.use_rel_pos and USE_CUSTOM_KERNEL and qkv.is_cuda
+                and self.rel_pos_h.shape[0] == 2 * H - 1 and self.rel_pos_w.shape[0] == 2 * W - 1
+                and ops.attn_supported(H * W, (H, W), hd, qkv.dtype))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        B, H, W, C = x.shape
+        nH = self.num_heads
+        hd = C // nH
+        qkv = self.qkv(x).reshape(B, H * W, 3, nH, hd)
+        if self._fused_ok(qkv, H, W, hd):
+            # strided (B, nH, N, hd) views of the token-major qkv buffer: no copies
+            q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+            out = ops.attn_relpos(q, k, v, self.rel_pos_h, self.rel_pos_w, (H, W), self.scale)
+            x = out.permute(0, 2, 1, 3).reshape(B, H, W, C)  # already token-major: a view
+            return self.proj(x)
+
+        q, k, v = qkv.permute(2, 0, 3, 1, 4).reshape(3, B * nH, H * W, hd).unbind(0)
+        if self.use_rel_pos:
+            rel_h, rel_w = add_decomposed_rel_pos(q, self.rel_pos_h, self.rel_pos_w, (H, W), (H, W))
+            rel_h = rel_h.view(B, nH, H * W, H, 1)
+            rel_w = rel_w.view(B, nH, H * W, 1, W)
+        q, k, v = (t.view(B, nH, H * W, hd) for t in (q, k, v))
+        if self.use_rel_pos:
+            x = _attention_rel_h_rel_w(q, k, v, rel_h, rel_w)
+        else:
+            x = F.scaled_dot_product_attention(q, k, v)
+        x = x.view(B, nH, H, W, hd).permute(0, 2, 3, 1, 4).reshape(B, H, W, C)
+        return self.proj(x)
+
+
+def window_partition(x: torch.Tensor, window_size: int) -> Tuple[torch.Tensor, Tuple[int, int]]:
+    """(B, H, W, C) -> ((B * nWindows, ws, ws, C), (Hp, Wp)), zero padding the
+    bottom and right edges up to a multiple of the window."""
+    B, H, W, C = x.shape
+    pad_h = (-H) % window_size
+    pad_w = (-W) % window_size
+    if pad_h or pad_w:
+        x = F.pad(x, (0, 0, 0, pad_w, 0, pad_h))
+    Hp, Wp = H + pad_h, W + pad_w
+    x = x.reshape(B, Hp // window_size, window_size, Wp // window_size, window_size, C)
+    windows = x.transpose(2, 3).reshape(-1, window_size, window_size, C)
+    return windows, (Hp, Wp)
+
+
+def window_unpartition(windows: torch.Tensor, window_size: int, pad_hw: Tuple[int, int],
+                       hw: Tuple[int, int]) -> torch.Tensor:
+    """Inverse of window_partition: back to (B, H, W, C) without the padding."""
+    Hp, Wp = pad_hw
+    H, W = hw
+    per_image = (Hp // window_size) * (Wp // window_size)
+    B = windows.shape[0] // per_image
+    x = windows.view(B, Hp // window_size, Wp // window_size, window_size, window_size, -1)
+    x = x.transpose(2, 3).reshape(B, Hp, Wp, -1)
+    if Hp > H or Wp > W:
+        x = x[:, :H, :W, :].contiguous()
+    return x
+
+
+def get_rel_pos(q_size: int, k_size: int, rel_pos: torch.Tensor) -> torch.Tensor:
+    """(q_size, k_size, C) relative-position embeddings gathered from an (L, C)
+    table, resizing the table linearly when L != 2*max(q_size, k_size) - 1."""
+    span = int(2 * max(q_size, k_size) - 1)
+    table = rel_pos
+    if table.shape[0] != span:
+        table = F.interpolate(table.t()[None], size=span, mode="linear")[0].t()
+    q_pos = torch.arange(q_size, device=rel_pos.device)[:, None] * max(k_size / q_size, 1.0)
+    k_pos = torch.arange(k_size, device=rel_pos.device)[None, :] * max(q_size / k_size, 1.0)
+    rel = (q_pos - k_pos) + (k_size - 1) * max(q_size / k_size, 1.0)
+    return table[rel.long()]
+
+
+def add_decomposed_rel_pos(
+    q: torch.Tensor,
+    rel_pos_h: torch.Tensor,
+    rel_pos_w: torch.Tensor,
+    q_size: Tuple[int, int],
+    k_size: Tuple[int, int],
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Bias factors for q (Bh, q_h*q_w, C): rel_h (Bh, q_h*q_w, k_h, 1) and
+    rel_w (Bh, q_h*q_w, 1, k_w)."""
+    q_h, q_w = q_size
+    k_h, k_w = k_size
+    Rh = get_rel_pos(q_h, k_h, rel_pos_h)
+    Rw = get_rel_pos(q_w, k_w, rel_pos_w)
+    Bh, _, dim = q.shape
+    grid = q.reshape(Bh, q_h, q_w, dim)
+    rel_h = torch.einsum("byxc,ykc->byxk", grid, Rh)
+    rel_w = torch.einsum("byxc,xkc->byxk", grid, Rw)
+    return (rel_h.reshape(Bh, q_h * q_w, k_h, 1), rel_w.reshape(Bh, q_h * q_w, 1, k_w))
+
+
+class PatchEmbed(nn.Module):
+    """Image to patch embedding: strided convolution, output (B, H, W, C)."""
+
+    def __init__(
+        self,
+        kernel_size: Tuple[int, int] = (16, 16),
+        stride: Tuple[int, int] = (16, 16),
+        padding: Tuple[int, int] = (0, 0),
+        in_chans: int = 3,
+        embed_dim: int = 768,
+    ) -> None:
+        super().__init__()
+        self.proj = nn.Conv2d(in_chans, embed_dim, kernel_size=kernel_size, stride=stride,
+                              padding=padding)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.proj(x).permute(0, 2, 3, 1)

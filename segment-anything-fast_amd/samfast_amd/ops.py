@@ -1,0 +1,159 @@
+"""Tensor-level wrappers over the C ABI: device pointers, strides and the current
+HIP stream are taken from torch tensors; all compute happens in libsamfast.so.
+
+Every function requires tensors on a GPU device and raises otherwise - there is
+no CPU or eager path behind these names.
+"""
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("samfast ops need GPU tensors (no CPU path exists)")
+
+
+def _bnhd_strides(t: torch.Tensor) -> Tuple[int, int, int]:
+    """(batch, head, token) element strides of a logical (B, nH, N, hd) tensor."""
+    if t.stride(3) != 1:
+        raise RuntimeError("samfast: the head_dim axis must be contiguous")
+    return t.stride(0), t.stride(1), t.stride(2)
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return _lib.SAMFAST_BF16
+    if t.dtype == torch.float16:
+        return _lib.SAMFAST_F16
+    raise RuntimeError(f"samfast: unsupported dtype {t.dtype}")
+
+
+def attn_supported(N: int, grid_hw: Tuple[int, int], hd: int, dtype: torch.dtype) -> bool:
+    """Shapes the HIP attention kernels cover (mirrors the checks in the library)."""
+    gh, gw = grid_hw
+    if dtype != torch.bfloat16 or hd not in (64, 80) or gh * gw != N:
+        return False
+    global_ok = gw == 64 and N % 128 == 0 and gh <= 64
+    window_ok = gh <= 15 and gw <= 16 and N <= 208
+    return global_ok or window_ok
+
+
+def attn_relpos(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                rel_pos_h: torch.Tensor, rel_pos_w: torch.Tensor,
+                grid_hw: Tuple[int, int], sm_scale: Optional[float] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """softmax(q k^T * scale + rel_h + rel_w) v with the bias computed in-kernel
+    from the (2S-1, hd) tables.  q, k, v: logical (B, nH, N, hd), any batch / head /
+    token strides (head_dim contiguous).  Returns (B, nH, N, hd) laid out
+    token-major, i.e. as a (B, N, nH*hd) buffer viewed head-major, unless `out`
+    is given."""
+    _require_gpu(q, k, v, rel_pos_h, rel_pos_w)
+    B, nH, N, hd = q.shape
+    gh, gw = grid_hw
+    if out is None:
+        out = torch.empty((B, N, nH, hd), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
+    rel_pos_h = rel_pos_h.contiguous()
+    rel_pos_w = rel_pos_w.contiguous()
+    if rel_pos_h.shape != (2 * gh - 1, hd) or rel_pos_w.shape != (2 * gw - 1, hd):
+        raise RuntimeError("samfast: relative-position tables must be (2*S-1, head_dim)")
+    if rel_pos_h.dtype != q.dtype or rel_pos_w.dtype != q.dtype:
+        rel_pos_h, rel_pos_w = rel_pos_h.to(q.dtype), rel_pos_w.to(q.dtype)
+    scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(hd)
+    lib = _lib.load()
+    code = lib.samfast_attn_relpos_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), rel_pos_h.data_ptr(), rel_pos_w.data_ptr(),
+        out.data_ptr(), B, nH, gh, gw, hd,
+        *_bnhd_strides(q), *_bnhd_strides(k), *_bnhd_strides(v), *_bnhd_strides(out),
+        _dtype_code(q), scale, _stream())
+    _lib.check(code, "attn_relpos_fwd")
+    return out
+
+
+def attn_relpos_bias(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                     rel_h: torch.Tensor, rel_w: torch.Tensor,
+                     sm_scale: Optional[float] = None,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Same attention with caller-computed bias factors rel_h (B, nH, N, gh) and
+    rel_w (B, nH, N, gw) (last axis contiguous).  Returns a contiguous
+    (B, nH, N, hd) tensor unless `out` is given."""
+    _require_gpu(q, k, v, rel_h, rel_w)
+    B, nH, N, hd = q.shape
+    gh, gw = rel_h.shape[-1], rel_w.shape[-1]
+    if rel_h.dtype != q.dtype or rel_w.dtype != q.dtype:
+        raise RuntimeError("samfast: bias factors must have the dtype of q")
+    if out is None:
+        out = torch.empty((B, nH, N, hd), dtype=q.dtype, device=q.device)
+    scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(hd)
+    lib = _lib.load()
+    code = lib.samfast_attn_relpos_bias_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), rel_h.data_ptr(), rel_w.data_ptr(),
+        out.data_ptr(), B, nH, gh, gw, hd,
+        *_bnhd_strides(q), *_bnhd_strides(k), *_bnhd_strides(v), *_bnhd_strides(out),
+        *_bnhd_strides(rel_h), *_bnhd_strides(rel_w),
+        _dtype_code(q), scale, _stream())
+    _lib.check(code, "attn_relpos_bias_fwd")
+    return out
+
+
+def quant_rowwise(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(M, K) bf16 (row stride free, K contiguous) -> (int8 (M, K), fp32 scales (M,))."""
+    _require_gpu(x)
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise RuntimeError("samfast: quant_rowwise needs a 2-D tensor with contiguous rows")
+    M, K = x.shape
+    xq = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    sx = torch.empty((M,), dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    code = lib.samfast_quant_rowwise_i8(
+        x.data_ptr(), x.stride(0), xq.data_ptr(), sx.data_ptr(), M, K, _dtype_code(x), _stream())
+    _lib.check(code, "quant_rowwise_i8")
+    return xq, sx
+
+
+def gemm_i8_i32(xq: torch.Tensor, wq: torch.Tensor) -> torch.Tensor:
+    """int8 (M, K) x int8 (N, K)^T -> int32 (M, N), exact."""
+    _require_gpu(xq, wq)
+    if xq.dtype != torch.int8 or wq.dtype != torch.int8:
+        raise RuntimeError("samfast: gemm_i8_i32 needs int8 operands")
+    if not (xq.is_contiguous() and wq.is_contiguous()) or xq.shape[1] != wq.shape[1]:
+        raise RuntimeError("samfast: gemm_i8_i32 needs contiguous (M, K) and (N, K)")
+    M, K = xq.shape
+    N = wq.shape[0]
+    acc = torch.empty((M, N), dtype=torch.int32, device=xq.device)
+    lib = _lib.load()
+    code = lib.samfast_gemm_i8_i32(xq.data_ptr(), wq.data_ptr(), acc.data_ptr(), M, N, K, _stream())
+    _lib.check(code, "gemm_i8_i32")
+    return acc
+
+
+def gemm_i8_scale_bias(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor,
+                       bias: Optional[torch.Tensor], out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bf16 (M, N) = (float(xq wq^T) * sx[:, None]) * sw[None, :] + bias."""
+    _require_gpu(xq, sx, wq, sw, bias)
+    if not (xq.is_contiguous() and wq.is_contiguous()) or xq.shape[1] != wq.shape[1]:
+        raise RuntimeError("samfast: gemm_i8_scale_bias needs contiguous (M, K) and (N, K)")
+    M, K = xq.shape
+    N = wq.shape[0]
+    if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != M or sw.numel() != N:
+        raise RuntimeError("samfast: scales must be fp32 of length M and N")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N):
+        raise RuntimeError("samfast: bias must be fp32 of length N")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=xq.device)
+    lib = _lib.load()
+    code = lib.samfast_gemm_i8_scale_bias(
+        xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
+        bias.data_ptr() if bias is not None else None, out.data_ptr(), out.stride(0),
+        M, N, K, _lib.SAMFAST_BF16, _stream())
+    _lib.check(code, "gemm_i8_scale_bias")
+    return out

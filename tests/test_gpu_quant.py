@@ -1,0 +1,108 @@
+"""GPU parity: dynamic int8 linear kernels (through the C ABI) against the CPU oracle.
+Integer results (int8 codes, int32 accumulators) must be bit-exact; so must the
+fp32-step-by-step epilogue and the scales."""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import linear_inputs
+from oracle import quant_linear as orq
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("M,K", [(1, 8), (7, 64), (300, 1280), (257, 5120), (64, 768), (33, 3072), (5, 8192)])
+def test_quant_rowwise_bit_exact(M, K):
+    from samfast_amd import ops
+    print(f"case quant M={M} K={K}", flush=True)
+    x, _, _ = linear_inputs(M, K, 8, seed=M + K)
+    if M > 2:
+        x[1] = 0  # an all-zero row: absmax floor
+    xq_ref, sx_ref = orq.quantize_rows_absmax(x)
+    xq, sx = ops.quant_rowwise(x.cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(sx.cpu().numpy(), sx_ref)
+    assert np.array_equal(xq.cpu().numpy(), xq_ref)
+
+
+def test_quant_rowwise_strided_rows():
+    from samfast_amd import ops
+    x, _, _ = linear_inputs(40, 256, 8, seed=9)
+    big = torch.zeros((40, 512), dtype=torch.bfloat16)
+    big[:, :256] = x
+    xq, sx = ops.quant_rowwise(big.cuda()[:, :256])
+    xq_ref, sx_ref = orq.quantize_rows_absmax(x)
+    assert np.array_equal(xq.cpu().numpy(), xq_ref) and np.array_equal(sx.cpu().numpy(), sx_ref)
+
+
+@pytest.mark.parametrize("M,N,K", [
+    (256, 256, 64), (1, 8, 64), (300, 264, 128), (513, 1280, 1280), (260, 3840, 1280),
+    (129, 1280, 5120), (4900, 768, 768), (31, 5120, 1280),
+])
+def test_gemm_i32_bit_exact(M, N, K):
+    from samfast_amd import ops
+    print(f"case gemm M={M} N={N} K={K}", flush=True)
+    g = torch.Generator().manual_seed(M * 7 + N * 3 + K)
+    xq = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+    wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    ref = orq.int8_gemm_i32(xq.numpy(), wq.numpy())
+    acc = ops.gemm_i8_i32(xq.cuda(), wq.cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(acc.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("M,N,K,with_bias", [(300, 264, 128, True), (777, 1280, 1280, True),
+                                             (130, 3840, 1280, False), (65, 1280, 5120, True)])
+def test_linear_end_to_end_bit_exact(M, N, K, with_bias):
+    """quantise -> GEMM -> scale/bias epilogue, every stage against the oracle."""
+    from samfast_amd import ops
+    from samfast_amd.quant import quantize_weight_per_channel
+    print(f"case linear M={M} N={N} K={K}", flush=True)
+    x, w, b = linear_inputs(M, K, N, seed=N + K)
+    bias = b if with_bias else None
+    wq_ref, sw_ref = orq.quantize_rows_absmax(w)
+    wq, sw = quantize_weight_per_channel(w)
+    assert np.array_equal(wq.numpy(), wq_ref) and np.array_equal(sw.numpy(), sw_ref)
+    y_ref = orq.dynamic_int8_linear(x, w, bias)
+    xq, sx = ops.quant_rowwise(x.cuda())
+    y = ops.gemm_i8_scale_bias(xq, sx, wq.cuda(), sw.cuda(),
+                               bias.float().cuda() if with_bias else None)
+    torch.cuda.synchronize()
+    assert torch.equal(y.cpu().view(torch.int16), y_ref.view(torch.int16))
+
+
+def test_full_size_checksum():
+    """Config-4 size (M = 65536, qkv 1280 -> 3840): int32 accumulators checked by a
+    size-independent property - column sums of acc equal (sum of x rows) . w, computed
+    exactly in int64 on the CPU - plus an exact row subset."""
+    from samfast_amd import ops
+    M, N, K = 65536, 3840, 1280
+    g = torch.Generator().manual_seed(4)
+    xq = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+    wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    acc = ops.gemm_i8_i32(xq.cuda(), wq.cuda())
+    col_sum = acc.to(torch.int64).sum(dim=0).cpu().numpy()
+    expect = xq.to(torch.int64).sum(dim=0).numpy() @ wq.to(torch.int64).numpy().T
+    assert np.array_equal(col_sum, expect)
+    rows = torch.randperm(M, generator=g)[:64]
+    sub = orq.int8_gemm_i64(xq[rows].numpy(), wq.numpy())
+    assert np.array_equal(acc[rows.cuda()].cpu().numpy().astype(np.int64), sub)
+
+
+def test_module_swap_forward():
+    """apply_dynamic_quant swaps Linears; forward equals the oracle's dynamic linear."""
+    from samfast_amd import apply_dynamic_quant
+    from samfast_amd.modeling import MLPBlock
+    torch.manual_seed(0)
+    mlp = MLPBlock(256, 1024).to(torch.bfloat16)
+    x = (torch.randn(3, 10, 256)).to(torch.bfloat16)
+    w1, b1 = mlp.lin1.weight.detach().clone(), mlp.lin1.bias.detach().clone()
+    w2, b2 = mlp.lin2.weight.detach().clone(), mlp.lin2.bias.detach().clone()
+    ref = orq.dynamic_int8_linear(
+        torch.nn.functional.gelu(orq.dynamic_int8_linear(x, w1, b1).float()).to(torch.bfloat16), w2, b2)
+    apply_dynamic_quant(mlp)
+    assert type(mlp.lin1).__name__ == "Int8DynamicLinear"
+    out = mlp.cuda()(x.cuda())
+    d = (out.float().cpu() - ref.float()).abs().max().item()
+    assert d <= 2e-2, d  # GELU on the GPU in bf16 vs fp32 on the CPU: not bit-exact
