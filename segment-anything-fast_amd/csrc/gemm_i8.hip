@@ -21,6 +21,10 @@
 // their X panels and the W matrix in that XCD's L2.
 #include "samfast_internal.hpp"
 
+// every fp32 step below is rounded on its own (no fused multiply-add), so results
+// can be reproduced bit for bit on a CPU
+#pragma clang fp contract(off)
+
 namespace samfast {
 
 constexpr int GBM = 256, GBN = 256, GBK = 64;
@@ -88,16 +92,16 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-  i32x4 sx_regs[4], sw_regs[4];
+  i32x4 stg_x[4], stg_w[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    sx_regs[i] = *reinterpret_cast<const i32x4*>(gx[i]);
-    sw_regs[i] = *reinterpret_cast<const i32x4*>(gw[i]);
+    stg_x[i] = *reinterpret_cast<const i32x4*>(gx[i]);
+    stg_w[i] = *reinterpret_cast<const i32x4*>(gw[i]);
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    *reinterpret_cast<i32x4*>(lds + lx[i]) = sx_regs[i];
-    *reinterpret_cast<i32x4*>(lds + lw[i]) = sw_regs[i];
+    *reinterpret_cast<i32x4*>(lds + lx[i]) = stg_x[i];
+    *reinterpret_cast<i32x4*>(lds + lw[i]) = stg_w[i];
   }
   __syncthreads();
 
@@ -111,8 +115,8 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmArgs a) {
     if (more) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        sx_regs[i] = *reinterpret_cast<const i32x4*>(gx[i] + (int64_t)(kt + 1) * GBK);
-        sw_regs[i] = *reinterpret_cast<const i32x4*>(gw[i] + (int64_t)(kt + 1) * GBK);
+        stg_x[i] = *reinterpret_cast<const i32x4*>(gx[i] + (int64_t)(kt + 1) * GBK);
+        stg_w[i] = *reinterpret_cast<const i32x4*>(gw[i] + (int64_t)(kt + 1) * GBK);
       }
     }
 #pragma unroll
@@ -133,8 +137,8 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmArgs a) {
       unsigned char* nxt = lds + ((kt + 1) & 1) * GSTAGE;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        *reinterpret_cast<i32x4*>(nxt + lx[i]) = sx_regs[i];
-        *reinterpret_cast<i32x4*>(nxt + lw[i]) = sw_regs[i];
+        *reinterpret_cast<i32x4*>(nxt + lx[i]) = stg_x[i];
+        *reinterpret_cast<i32x4*>(nxt + lw[i]) = stg_w[i];
       }
     }
     __syncthreads();
@@ -167,9 +171,9 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(GemmArgs a) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             // three separately rounded fp32 operations (no fused multiply-add)
-            float t = __fmul_rn((float)acc[i][j][r], s);
-            t = __fmul_rn(t, swv[j]);
-            y[j] = __fadd_rn(t, bv4[j]);
+            float t = (float)acc[i][j][r] * s;
+            t = t * swv[j];
+            y[j] = t + bv4[j];
           }
           u32x2 o = {pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3])};
           *reinterpret_cast<u32x2*>(reinterpret_cast<unsigned short*>(a.out) + (int64_t)m * a.ldo + nc) = o;

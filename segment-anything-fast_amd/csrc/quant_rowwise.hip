@@ -6,6 +6,10 @@
 // 2 bytes read + 1 byte written per element plus 4 bytes of scale per row.
 #include "samfast_internal.hpp"
 
+// every fp32 step below is rounded on its own (no fused multiply-add), so results
+// can be reproduced bit for bit on a CPU
+#pragma clang fp contract(off)
+
 namespace samfast {
 
 constexpr int kQuantWavesPerBlock = 4;
@@ -37,7 +41,7 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
 
-  const float scale = __fdiv_rn(fmaxf(amax, 1e-5f), 127.0f);
+  const float scale = fmaxf(amax, 1e-5f) / 127.0f;
   if (lane == 0) sx[row] = scale;
 
   u32x2* dst = reinterpret_cast<u32x2*>(xq + row * (int64_t)K);
@@ -51,8 +55,8 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
         const float lo = bf16_lo_to_f32(buf[i][j]);
         const float hi = bf16_hi_to_f32(buf[i][j]);
         // IEEE division, then round half to even, then clamp
-        const int qlo = (int)fminf(fmaxf(rintf(__fdiv_rn(lo, scale)), -127.f), 127.f);
-        const int qhi = (int)fminf(fmaxf(rintf(__fdiv_rn(hi, scale)), -127.f), 127.f);
+        const int qlo = (int)fminf(fmaxf(rintf(lo / scale), -127.f), 127.f);
+        const int qhi = (int)fminf(fmaxf(rintf(hi / scale), -127.f), 127.f);
         const int e = 2 * j;  // element index inside the chunk
         packed[e >> 2] |= ((unsigned int)(qlo & 0xff)) << (8 * (e & 3));
         packed[(e + 1) >> 2] |= ((unsigned int)(qhi & 0xff)) << (8 * ((e + 1) & 3));
