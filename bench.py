@@ -1,0 +1,173 @@
+#!/usr/bin/env python3
+"""Benchmark of the SAM ViT image-encoder hot path on one MI355X.
+
+One step = one forward of the ViT-H image encoder over a batch of 16 synthetic
+1024x1024 images (bf16 activations, rel-pos attention on the HIP flash kernels,
+all four Linears of every block on the dynamic-int8 HIP kernels), inputs and
+weights resident in HBM before the timed region.
+
+Prints ONE JSON line: images/s plus
+  roofline      the dominant kernel (by time inside a step) against its bound,
+                from per-launch event timings of an instrumented step;
+  kernels       the same figures for every hand-written kernel in the step;
+  gpu_baseline  the same encoder through PyTorch-ROCm bf16 SDPA + bf16 Linear;
+  cpu_baseline  the CPU oracle (the reference's eager route) on one image.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT / "segment-anything-fast_amd"))
+sys.path.insert(0, str(ROOT))
+
+PEAK = {"op": ("mfma", 5.0e15, "TOP/s"),       # int8 dense MFMA
+        "flop": ("mfma", 2.5e15, "TFLOP/s"),   # bf16 dense MFMA
+        "byte": ("hbm", 8.0e12, "GB/s")}       # HBM3E
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=10)
+    p.add_argument("--warmup", type=int, default=3)
+    p.add_argument("--model", default="vit_h", choices=["vit_h", "vit_l", "vit_b"])
+    p.add_argument("--batch", type=int, default=16)
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--no-gpu-baseline", action="store_true")
+    p.add_argument("--bf16-linears", action="store_true", help="keep nn.Linear (attention kernels only)")
+    return p.parse_args()
+
+
+def time_steps(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def kernel_table(summary):
+    rows = {}
+    for name, d in summary.items():
+        bound, peak, unit = PEAK[d["unit"]]
+        sec = d["ms"] * 1e-3
+        rate = d["work"] / sec if sec > 0 else 0.0
+        scale = 1e-9 if unit == "GB/s" else 1e-12
+        rows[name] = {
+            "launches": d["launches"], "ms_total": round(d["ms"], 3),
+            "avg_us": round(1e3 * d["ms"] / d["launches"], 2),
+            "bound": bound, "achieved": round(rate * scale, 2), "peak": peak * scale,
+            "unit": unit, "frac": round(rate / peak, 4),
+        }
+    return rows
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives exist on this path); "
+              "use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from samfast_amd import apply_dynamic_quant, flash_4, ops
+    from samfast_amd.build_sam import build_image_encoder
+    from samfast_amd.synthetic import init_encoder_weights, make_images
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    enc = build_image_encoder(args.model)
+    sd_fp32 = {k: v.clone() for k, v in init_encoder_weights(enc, seed=0).items()}
+    enc = enc.eval().to(torch.bfloat16).to(dev)
+    if not args.bf16_linears:
+        apply_dynamic_quant(enc)
+    images = make_images(args.batch, seed=1).to(torch.bfloat16).to(dev)
+
+    with torch.no_grad():
+        step = lambda: enc(images)
+        sec = time_steps(step, args.steps, args.warmup)
+        out = step()
+        finite = bool(torch.isfinite(out.float()).all())
+
+        # instrumented step: events around every hand-written kernel launch
+        with ops.record_launches() as rec:
+            step()
+        kernels = kernel_table(rec.summary())
+
+    dominant = max(kernels, key=lambda n: kernels[n]["ms_total"])
+    dk = kernels[dominant]
+    roofline = {"kernel": dominant, "bound": dk["bound"], "achieved": dk["achieved"],
+                "peak": dk["peak"], "unit": dk["unit"], "frac": dk["frac"], "traffic": None,
+                "avg_us": dk["avg_us"], "launches_per_step": dk["launches"]}
+
+    result = {
+        "metric": "images/s ViT-H encoder bs16 1024^2" if (args.model, args.batch) == ("vit_h", 16)
+        else f"images/s {args.model} encoder bs{args.batch} 1024^2",
+        "value": round(args.batch / sec, 3), "unit": "images/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 attention + int8 linears (int32 accumulate)" if not args.bf16_linears else "bf16",
+        "data": "synthetic (seeded uniform images, random-init weights)",
+        "config": {"workload": f"SAM {args.model} image encoder forward, batch {args.batch}, "
+                               "1024x1024, rel-pos attention + dynamic int8 linears",
+                   "batch": args.batch, "image": 1024},
+        "output_finite": finite,
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+
+    if not args.no_gpu_baseline:
+        # same weights, PyTorch-ROCm eager: bf16 nn.Linear + SDPA with a materialised bias
+        base = build_image_encoder(args.model)
+        base.load_state_dict(sd_fp32)
+        base = base.eval().to(torch.bfloat16).to(dev)
+        flash_4.USE_CUSTOM_KERNEL = False
+        try:
+            with torch.no_grad():
+                bsec = time_steps(lambda: base(images), 3, 1)
+                ref = base(images)
+            cos = torch.nn.functional.cosine_similarity(
+                out.float().flatten(1), ref.float().flatten(1), dim=1).min().item()
+        finally:
+            flash_4.USE_CUSTOM_KERNEL = True
+        result["gpu_baseline"] = {"what": "same encoder, PyTorch-ROCm eager bf16 SDPA(attn_mask) + bf16 nn.Linear",
+                                  "value": round(args.batch / bsec, 3), "unit": "images/s",
+                                  "ms_per_step": round(bsec * 1e3, 3),
+                                  "speedup": round(bsec / sec, 3),
+                                  "min_cosine_vs_this_path": round(cos, 6)}
+        del base, ref
+        torch.cuda.empty_cache()
+
+    if not args.no_cpu_baseline:
+        from oracle import image_encoder as oe
+        cfg = {"vit_h": oe.VIT_H, "vit_l": oe.VIT_L, "vit_b": oe.VIT_B}[args.model]
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+        torch.set_num_threads(cores)
+        x1 = make_images(1, seed=1)
+        with torch.no_grad():
+            t0 = time.perf_counter()
+            oe.encoder_forward(sd_fp32, x1, cfg, use_sdpa=True)
+            csec = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": round(1.0 / csec, 4), "unit": "images/s", "cores": cores,
+                                  "kind": "port",
+                                  "sample": f"1 image through the whole {args.model} encoder, fp32 eager "
+                                            "(SDPA with materialised bias, fp32 Linear), one run"}
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -69,7 +69,8 @@ def layer_norm_2d(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps
 
 
 def block_forward(sd: Dict[str, torch.Tensor], prefix: str, x: torch.Tensor,
-                  cfg: EncoderConfig, window_size: int, linear=F.linear) -> torch.Tensor:
+                  cfg: EncoderConfig, window_size: int, linear=F.linear,
+                  use_sdpa: bool = False) -> torch.Tensor:
     """One transformer block on (B, H, W, C); image_encoder.py:167-183."""
     C = cfg.embed_dim
     p = lambda name: sd[prefix + name]
@@ -81,6 +82,7 @@ def block_forward(sd: Dict[str, torch.Tensor], prefix: str, x: torch.Tensor,
     y = ra.attention_forward(
         y, p("attn.qkv.weight"), p("attn.qkv.bias"), p("attn.proj.weight"), p("attn.proj.bias"),
         p("attn.rel_pos_h"), p("attn.rel_pos_w"), cfg.num_heads, linear=linear,
+        use_sdpa=use_sdpa,
     )
     if window_size > 0:
         y = ra.window_unpartition(y, window_size, pad_hw, (H, W))
@@ -93,12 +95,15 @@ def block_forward(sd: Dict[str, torch.Tensor], prefix: str, x: torch.Tensor,
 
 
 def encoder_forward(sd: Dict[str, torch.Tensor], images: torch.Tensor, cfg: EncoderConfig,
-                    linear=F.linear) -> torch.Tensor:
+                    linear=F.linear, use_sdpa: bool = False) -> torch.Tensor:
     """(B, 3, 1024, 1024) normalised images -> (B, 256, 64, 64) embeddings.
 
     `linear(x, w, b)` is used for the four Linears of every block (qkv, proj,
     lin1, lin2) - pass oracle.quant_linear.dynamic_int8_linear for the
     quantised path.  Patch embedding and neck are convolutions and stay float.
+    use_sdpa=True routes attention through F.scaled_dot_product_attention with a
+    materialised bias, which is what the reference executes on a CPU
+    (flash_4.py:368-370); the default writes the softmax out.
     """
     x = F.conv2d(images, sd["patch_embed.proj.weight"], sd["patch_embed.proj.bias"],
                  stride=cfg.patch_size)
@@ -107,7 +112,7 @@ def encoder_forward(sd: Dict[str, torch.Tensor], images: torch.Tensor, cfg: Enco
         x = x + sd["pos_embed"]
     for i in range(cfg.depth):
         ws = 0 if i in cfg.global_attn_indexes else cfg.window_size
-        x = block_forward(sd, f"blocks.{i}.", x, cfg, ws, linear)
+        x = block_forward(sd, f"blocks.{i}.", x, cfg, ws, linear, use_sdpa)
     x = x.permute(0, 3, 1, 2)
     x = F.conv2d(x, sd["neck.0.weight"])
     x = layer_norm_2d(x, sd["neck.1.weight"], sd["neck.1.bias"])

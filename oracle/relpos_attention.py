@@ -122,6 +122,16 @@ def attention_rel_h_rel_w(
     return torch.matmul(probs, vc)
 
 
+def attention_rel_h_rel_w_sdpa(q, k, v, rel_h, rel_w) -> torch.Tensor:
+    """The same function through the library call the reference itself makes on
+    a CPU (flash_4.py:368-370): materialise rel_h + rel_w as an additive mask and
+    hand it to F.scaled_dot_product_attention.  Used as the timed CPU baseline and
+    as the cross-check of attention_rel_h_rel_w."""
+    B, nH, N, _ = q.shape
+    bias = (rel_h + rel_w).reshape(B, nH, N, rel_h.shape[3] * rel_w.shape[4])
+    return F.scaled_dot_product_attention(q, k, v, attn_mask=bias)
+
+
 def attention_from_tables(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -130,6 +140,7 @@ def attention_from_tables(
     rel_pos_w: torch.Tensor,
     grid_hw: Tuple[int, int],
     compute_dtype: torch.dtype = torch.float32,
+    use_sdpa: bool = False,
 ) -> torch.Tensor:
     """Bias from the (2S-1, hd) tables, then attention_rel_h_rel_w.
 
@@ -142,6 +153,9 @@ def attention_from_tables(
     )
     rel_h = rel_h.reshape(B, nH, N, grid_hw[0], 1)
     rel_w = rel_w.reshape(B, nH, N, 1, grid_hw[1])
+    if use_sdpa:
+        return attention_rel_h_rel_w_sdpa(
+            q.to(compute_dtype), k.to(compute_dtype), v.to(compute_dtype), rel_h, rel_w)
     return attention_rel_h_rel_w(q, k, v, rel_h, rel_w, compute_dtype)
 
 
@@ -185,6 +199,7 @@ def attention_forward(
     rel_pos_w: torch.Tensor,
     num_heads: int,
     linear=F.linear,
+    use_sdpa: bool = False,
 ) -> torch.Tensor:
     """Attention.forward of image_encoder.py:225-253 on (B, H, W, C) tokens.
 
@@ -197,7 +212,8 @@ def attention_forward(
     qkv = linear(x.reshape(B, N, C), qkv_weight, qkv_bias)
     qkv = qkv.reshape(B, N, 3, num_heads, hd).permute(2, 0, 3, 1, 4)  # (3, B, nH, N, hd)
     q, k, v = qkv[0], qkv[1], qkv[2]
-    out = attention_from_tables(q, k, v, rel_pos_h, rel_pos_w, (H, W), compute_dtype=q.dtype)
+    out = attention_from_tables(q, k, v, rel_pos_h, rel_pos_w, (H, W), compute_dtype=q.dtype,
+                                use_sdpa=use_sdpa)
     out = out.permute(0, 2, 1, 3).reshape(B, N, C)  # heads back into channels
     out = linear(out, proj_weight, proj_bias)
     return out.reshape(B, H, W, C)

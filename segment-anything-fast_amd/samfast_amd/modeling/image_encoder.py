@@ -22,7 +22,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .. import ops
-from ..flash_4 import USE_CUSTOM_KERNEL, _attention_rel_h_rel_w
+from .. import flash_4
+from ..flash_4 import _attention_rel_h_rel_w
 from .common import LayerNorm2d, MLPBlock
 
 
@@ -147,7 +148,7 @@ class Attention(nn.Module):
             self.rel_pos_w = nn.Parameter(torch.zeros(2 * input_size[1] - 1, head_dim))
 
     def _fused_ok(self, qkv: torch.Tensor, H: int, W: int, hd: int) -> bool:
-        return (self.use_rel_pos and USE_CUSTOM_KERNEL and qkv.is_cuda
+        return (self.use_rel_pos and flash_4.USE_CUSTOM_KERNEL and qkv.is_cuda
                 and self.rel_pos_h.shape[0] == 2 * H - 1 and self.rel_pos_w.shape[0] == 2 * W - 1
                 and ops.attn_supported(H * W, (H, W), hd, qkv.dtype))
 

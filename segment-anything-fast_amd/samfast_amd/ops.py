@@ -17,6 +17,52 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+# Optional per-launch timing: while a list is installed with record_launches(), every
+# kernel launch is bracketed by two events on the stream it is enqueued on and
+# (kernel, algorithmic work, unit, start, end) is appended.  Used by the benchmark to
+# get per-kernel durations of a real encoder step; off (None) otherwise.
+_launch_log = None
+
+
+class record_launches:
+    def __init__(self):
+        self.entries = []
+
+    def __enter__(self):
+        global _launch_log
+        self._prev, _launch_log = _launch_log, self.entries
+        return self
+
+    def __exit__(self, *exc):
+        global _launch_log
+        _launch_log = self._prev
+        return False
+
+    def summary(self):
+        """{kernel: dict(launches, work, unit, ms)} after synchronising."""
+        torch.cuda.synchronize()
+        out = {}
+        for name, work, unit, e0, e1 in self.entries:
+            d = out.setdefault(name, dict(launches=0, work=0.0, unit=unit, ms=0.0))
+            d["launches"] += 1
+            d["work"] += work
+            d["ms"] += e0.elapsed_time(e1)
+        return out
+
+
+def _timed(name: str, work: float, unit: str, launch):
+    log = _launch_log
+    if log is None:
+        return launch()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    code = launch()
+    e1.record()
+    log.append((name, work, unit, e0, e1))
+    return code
+
+
 def _require_gpu(*tensors: torch.Tensor) -> None:
     for t in tensors:
         if t is not None and not t.is_cuda:
@@ -70,11 +116,13 @@ def attn_relpos(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         rel_pos_h, rel_pos_w = rel_pos_h.to(q.dtype), rel_pos_w.to(q.dtype)
     scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(hd)
     lib = _lib.load()
-    code = lib.samfast_attn_relpos_fwd(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), rel_pos_h.data_ptr(), rel_pos_w.data_ptr(),
-        out.data_ptr(), B, nH, gh, gw, hd,
-        *_bnhd_strides(q), *_bnhd_strides(k), *_bnhd_strides(v), *_bnhd_strides(out),
-        _dtype_code(q), scale, _stream())
+    code = _timed(
+        "attn_global" if gw == 64 else "attn_window", 4.0 * B * nH * N * N * hd, "flop",
+        lambda: lib.samfast_attn_relpos_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), rel_pos_h.data_ptr(), rel_pos_w.data_ptr(),
+            out.data_ptr(), B, nH, gh, gw, hd,
+            *_bnhd_strides(q), *_bnhd_strides(k), *_bnhd_strides(v), *_bnhd_strides(out),
+            _dtype_code(q), scale, _stream()))
     _lib.check(code, "attn_relpos_fwd")
     return out
 
@@ -95,12 +143,14 @@ def attn_relpos_bias(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         out = torch.empty((B, nH, N, hd), dtype=q.dtype, device=q.device)
     scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(hd)
     lib = _lib.load()
-    code = lib.samfast_attn_relpos_bias_fwd(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), rel_h.data_ptr(), rel_w.data_ptr(),
-        out.data_ptr(), B, nH, gh, gw, hd,
-        *_bnhd_strides(q), *_bnhd_strides(k), *_bnhd_strides(v), *_bnhd_strides(out),
-        *_bnhd_strides(rel_h), *_bnhd_strides(rel_w),
-        _dtype_code(q), scale, _stream())
+    code = _timed(
+        "attn_global_bias" if gw == 64 else "attn_window_bias", 4.0 * B * nH * N * N * hd, "flop",
+        lambda: lib.samfast_attn_relpos_bias_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), rel_h.data_ptr(), rel_w.data_ptr(),
+            out.data_ptr(), B, nH, gh, gw, hd,
+            *_bnhd_strides(q), *_bnhd_strides(k), *_bnhd_strides(v), *_bnhd_strides(out),
+            *_bnhd_strides(rel_h), *_bnhd_strides(rel_w),
+            _dtype_code(q), scale, _stream()))
     _lib.check(code, "attn_relpos_bias_fwd")
     return out
 
@@ -114,8 +164,11 @@ def quant_rowwise(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     xq = torch.empty((M, K), dtype=torch.int8, device=x.device)
     sx = torch.empty((M,), dtype=torch.float32, device=x.device)
     lib = _lib.load()
-    code = lib.samfast_quant_rowwise_i8(
-        x.data_ptr(), x.stride(0), xq.data_ptr(), sx.data_ptr(), M, K, _dtype_code(x), _stream())
+    code = _timed(
+        "quant_rowwise", 3.0 * M * K + 4.0 * M, "byte",
+        lambda: lib.samfast_quant_rowwise_i8(
+            x.data_ptr(), x.stride(0), xq.data_ptr(), sx.data_ptr(), M, K, _dtype_code(x),
+            _stream()))
     _lib.check(code, "quant_rowwise_i8")
     return xq, sx
 
@@ -131,7 +184,10 @@ def gemm_i8_i32(xq: torch.Tensor, wq: torch.Tensor) -> torch.Tensor:
     N = wq.shape[0]
     acc = torch.empty((M, N), dtype=torch.int32, device=xq.device)
     lib = _lib.load()
-    code = lib.samfast_gemm_i8_i32(xq.data_ptr(), wq.data_ptr(), acc.data_ptr(), M, N, K, _stream())
+    code = _timed(
+        "gemm_i8_i32", 2.0 * M * N * K, "op",
+        lambda: lib.samfast_gemm_i8_i32(xq.data_ptr(), wq.data_ptr(), acc.data_ptr(), M, N, K,
+                                        _stream()))
     _lib.check(code, "gemm_i8_i32")
     return acc
 
@@ -151,9 +207,11 @@ def gemm_i8_scale_bias(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw:
     if out is None:
         out = torch.empty((M, N), dtype=torch.bfloat16, device=xq.device)
     lib = _lib.load()
-    code = lib.samfast_gemm_i8_scale_bias(
-        xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
-        bias.data_ptr() if bias is not None else None, out.data_ptr(), out.stride(0),
-        M, N, K, _lib.SAMFAST_BF16, _stream())
+    code = _timed(
+        "gemm_i8_scale_bias", 2.0 * M * N * K, "op",
+        lambda: lib.samfast_gemm_i8_scale_bias(
+            xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
+            bias.data_ptr() if bias is not None else None, out.data_ptr(), out.stride(0),
+            M, N, K, _lib.SAMFAST_BF16, _stream()))
     _lib.check(code, "gemm_i8_scale_bias")
     return out
