@@ -1,0 +1,129 @@
+"""CPU-side checks of the boundary: the C-ABI library loads and exports every symbol
+include/samfast.h declares (no compute calls without a GPU); the Python mirror keeps the
+reference's names and signatures; the product refuses to run without its kernels."""
+
+import ctypes
+import inspect
+import re
+from pathlib import Path
+
+import pytest
+import torch
+import torch.nn as nn
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def _header_functions():
+    text = (ROOT / "include" / "samfast.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(samfast_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from samfast_amd import _lib
+    names = _header_functions()
+    assert len(names) >= 8
+    lib = ctypes.CDLL(str(_lib.lib_path()))
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(_lib.EXPORTED_SYMBOLS) == names
+    loaded = _lib.load()
+    assert loaded.samfast_version() == 1
+    assert loaded.samfast_arch() == b"gfx950"
+
+
+def test_argument_validation_without_gpu():
+    """Validation runs on the host before any launch, so error codes are testable here."""
+    from samfast_amd import _lib
+    lib = _lib.load()
+    rc = lib.samfast_gemm_i8_i32(None, None, None, 16, 16, 64, None)
+    assert rc == -1 and b"null pointer" in lib.samfast_last_error()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    p += (-p) % 16
+    rc = lib.samfast_gemm_i8_i32(p, p, p, 16, 16, 100, None)
+    assert rc == -1 and b"multiple of 64" in lib.samfast_last_error()
+    rc = lib.samfast_quant_rowwise_i8(p, 12, p, p, 4, 12, 0, None)
+    assert rc == -1 and b"multiple of 8" in lib.samfast_last_error()
+    strides = [0] * 12
+    rc = lib.samfast_attn_relpos_fwd(p, p, p, p, p, p, 1, 1, 10, 10, 48, *strides, 0, 0.125, None)
+    assert rc == -2 and b"head_dim" in lib.samfast_last_error()
+    rc = lib.samfast_attn_relpos_fwd(p, p, p, p, p, p, 1, 1, 20, 20, 64, *([64] * 12), 0, 0.125, None)
+    assert rc == -2 and b"neither" in lib.samfast_last_error()
+    rc = lib.samfast_attn_relpos_fwd(p, p, p, p, p, p, 1, 1, 14, 14, 64, *([64] * 12), 1, 0.125, None)
+    assert rc == -2  # fp16 not built
+
+
+def test_ops_refuse_cpu_tensors():
+    from samfast_amd import ops
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.quant_rowwise(x)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.gemm_i8_i32(torch.zeros(4, 64, dtype=torch.int8), torch.zeros(8, 64, dtype=torch.int8))
+
+
+def test_registry_surface():
+    import samfast_amd
+    for reg in (samfast_amd.sam_model_registry, samfast_amd.sam_model_fast_registry):
+        assert set(reg) == {"default", "vit_h", "vit_l", "vit_b"}
+    sig = inspect.signature(samfast_amd.build_sam_fast_vit_h)
+    assert list(sig.parameters) == ["checkpoint", "compile_mode", "dtype"]
+    assert sig.parameters["compile_mode"].default == "max-autotune"
+    assert sig.parameters["dtype"].default == torch.bfloat16
+    sam = samfast_amd.sam_model_fast_registry["vit_b"]()
+    assert next(sam.image_encoder.parameters()).dtype == torch.bfloat16 and not sam.image_encoder.training
+    pred = samfast_amd.SamPredictor(sam)
+    assert pred.is_image_set is False
+    img = torch.zeros(1, 3, 512, 1024)
+    assert sam.preprocess(img).shape == (1, 3, 1024, 1024)
+
+
+def test_module_signatures_follow_reference():
+    from samfast_amd.modeling import Attention, Block, ImageEncoderViT, MLPBlock
+    assert list(inspect.signature(Attention.__init__).parameters)[1:] == [
+        "dim", "num_heads", "qkv_bias", "use_rel_pos", "rel_pos_zero_init", "input_size"]
+    assert list(inspect.signature(MLPBlock.__init__).parameters)[1:] == ["embedding_dim", "mlp_dim", "act"]
+    assert list(inspect.signature(Block.__init__).parameters)[1:] == [
+        "dim", "num_heads", "mlp_ratio", "qkv_bias", "norm_layer", "act_layer", "use_rel_pos",
+        "rel_pos_zero_init", "window_size", "input_size"]
+    att = Attention(64, 2, use_rel_pos=True, input_size=(14, 14))
+    assert {n for n, _ in att.named_parameters()} == {
+        "qkv.weight", "qkv.bias", "proj.weight", "proj.bias", "rel_pos_h", "rel_pos_w"}
+    assert att.rel_pos_h.shape == (27, 32)
+    enc_sig = inspect.signature(ImageEncoderViT.__init__)
+    assert enc_sig.parameters["window_size"].default == 0 and enc_sig.parameters["embed_dim"].default == 768
+
+
+def test_swap_helpers():
+    from samfast_amd import Int8DynamicLinear, apply_dynamic_quant
+    from samfast_amd.tools import replace_with_custom_fn_if_matches_filter
+    from samfast_amd.modeling import Block
+    blk = Block(64, 2, use_rel_pos=True, window_size=3, input_size=(8, 8))
+    seen = []
+    replace_with_custom_fn_if_matches_filter(
+        blk, lambda m: m, lambda m, fqn: (seen.append(fqn) or False))
+    assert {"norm1", "attn", "attn.qkv", "attn.proj", "norm2", "mlp", "mlp.lin1", "mlp.lin2", "mlp.act"} <= set(seen)
+    w = blk.mlp.lin1.weight.detach().clone()
+    apply_dynamic_quant(blk, lambda m, fqn: fqn.startswith("mlp."))
+    assert isinstance(blk.mlp.lin1, Int8DynamicLinear) and isinstance(blk.mlp.lin2, Int8DynamicLinear)
+    assert isinstance(blk.attn.qkv, nn.Linear)
+    assert blk.mlp.lin1.wq.dtype == torch.int8 and blk.mlp.lin1.sw.dtype == torch.float32
+    assert (blk.mlp.lin1.weight - w).abs().max() <= blk.mlp.lin1.sw.max() * 0.5001
+    blk = blk.to(torch.bfloat16)  # scales and integer weights survive a dtype cast untouched
+    assert blk.mlp.lin1.sw.dtype == torch.float32 and blk.mlp.lin1.wq.dtype == torch.int8
+    with pytest.raises(RuntimeError, match="GPU"):
+        blk.mlp(torch.zeros(1, 8, 8, 64, dtype=torch.bfloat16))  # no CPU route for the int8 path
+
+
+def test_composite_cpu_route_is_the_reference_fallback():
+    """fp32 / CPU inputs take the eager SDPA route exactly as flash_4.py:368-370."""
+    from samfast_amd.flash_4 import _attention_rel_h_rel_w
+    from oracle import relpos_attention as ora
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(1, 2, 196, 64, generator=g) for _ in range(3))
+    rel_h, rel_w = torch.randn(1, 2, 196, 14, 1, generator=g), torch.randn(1, 2, 196, 1, 14, generator=g)
+    got = _attention_rel_h_rel_w(q, k, v, rel_h, rel_w)
+    assert torch.allclose(got, ora.attention_rel_h_rel_w(q, k, v, rel_h, rel_w), atol=1e-5)
+    assert hasattr(torch.ops.customflash, "custom_flash_aligned")
