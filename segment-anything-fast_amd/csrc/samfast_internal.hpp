@@ -51,8 +51,10 @@ SF_DEVICE unsigned int f32_to_bf16_bits(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);
   return u >> 16;
 }
+// two fp32 -> packed bf16 pair, round to nearest even, one v_cvt_pk_bf16_f32
 SF_DEVICE unsigned int pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  const f32x2 v = {lo, hi};
+  return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, bf16x2));
 }
 
 SF_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
