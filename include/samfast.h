@@ -128,6 +128,43 @@ int samfast_gemm_i8_scale_bias(
     const float* bias, void* y, int64_t ldy,
     int64_t M, int N, int K, int dtype, void* stream);
 
+/*
+ * LayerNorm over each row followed by the per-row int8 quantiser, with an optional
+ * row gather: output row r is computed from source row src_row[r] of x (src_row NULL =
+ * identity); src_row[r] < 0 yields an all-zero row with scale 1e-5/127.
+ *   y = (x - mean) / sqrt(var + eps) * gamma + beta   (fp32, biased variance, rounded
+ *   to `dtype` as a separate LayerNorm would store it), then quantised as above.
+ * One launch for norm1 + window_partition (zero padding to the window multiple) + the
+ * qkv Linear's activation quantiser (modeling/image_encoder.py:169-173), or norm2 +
+ * lin1's quantiser (:181).  gamma, beta: K values of type `dtype`.
+ */
+int samfast_layernorm_quant_i8(
+    const void* x, int64_t ldx, const void* gamma, const void* beta, float eps,
+    const int32_t* src_row, int8_t* xq, float* sx,
+    int64_t M, int K, int dtype, void* stream);
+
+/* epilogues of samfast_gemm_i8_fused */
+#define SAMFAST_EPILOGUE_NONE 0      /* same as samfast_gemm_i8_scale_bias */
+#define SAMFAST_EPILOGUE_GELU 1      /* y = gelu_erf(bf16(linear))                 */
+#define SAMFAST_EPILOGUE_RESIDUAL 2  /* y[dst] = bf16(linear) + residual[dst]      */
+
+/*
+ * samfast_gemm_i8_scale_bias with a fused tail:
+ *   GELU      exact-erf GELU of the bf16-rounded Linear output - lin1 followed by
+ *             act() in MLPBlock.forward (modeling/common.py:26);
+ *   RESIDUAL  adds `residual` (bf16, row stride ld_res) and scatters rows: GEMM row m
+ *             is written to output row dst_row[m] (NULL = identity, < 0 = dropped) and
+ *             the residual is read at that same output row.  With the inverse window
+ *             map this is proj + window_unpartition + `shortcut + x`
+ *             (modeling/image_encoder.py:176-180); with the identity map it is lin2 +
+ *             `x + mlp(...)` (:181).  y and residual may be the same buffer.
+ */
+int samfast_gemm_i8_fused(
+    const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
+    const float* bias, void* y, int64_t ldy,
+    int64_t M, int N, int K, int dtype, int epilogue,
+    const void* residual, int64_t ld_res, const int32_t* dst_row, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -35,7 +35,7 @@ namespace samfast {
 constexpr int GBN = 256, GBK = 64;
 constexpr int GLD = GBK + 16;  // padded LDS row, bytes
 
-enum { EPI_I32 = 0, EPI_SCALE_BIAS_BF16 = 1 };
+enum { EPI_I32 = 0, EPI_SCALE_BIAS_BF16 = 1, EPI_GELU_BF16 = 2, EPI_RESIDUAL_BF16 = 3 };
 
 struct GemmArgs {
   const int8_t* x;
@@ -47,7 +47,26 @@ struct GemmArgs {
   int64_t ldo;
   int M, N, K;
   int tiles_m, tiles_n;
+  const unsigned short* residual;  // EPI_RESIDUAL: (rows, N) bf16, row stride ld_res
+  int64_t ld_res;
+  const int32_t* dst_row;          // EPI_RESIDUAL: output row per GEMM row, -1 = drop; may be null
 };
+
+// x * Phi(x) with Phi from the Abramowitz-Stegun 7.1.26 erfc polynomial (|error| <
+// 1.5e-7), evaluated as erfc on the negative side so the tail keeps its relative accuracy.
+SF_DEVICE float gelu_erf(float x) {
+#pragma clang fp contract(fast)  // an approximation anyway: let the polynomial use FMAs
+  const float z = fabsf(x) * 0.70710678118654752f;
+  const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
+  float poly = 1.061405429f;
+  poly = poly * t + -1.453152027f;
+  poly = poly * t + 1.421413741f;
+  poly = poly * t + -0.284496736f;
+  poly = poly * t + 0.254829592f;
+  const float half_erfc = 0.5f * poly * t * __builtin_amdgcn_exp2f(-1.4426950408889634f * z * z);
+  const float phi = x >= 0.f ? 1.0f - half_erfc : half_erfc;
+  return x * phi;
+}
 
 template <int EPI, int TM>
 __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArgs a) {
@@ -211,11 +230,41 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
   f32x4 bv4 = {0.f, 0.f, 0.f, 0.f};
   if (a.bias) bv4 = *reinterpret_cast<const f32x4*>(a.bias + nc);
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TM; ++i) {
+    // EPI_RESIDUAL: output rows (possibly remapped) and the residual values of this
+    // group of 16 rows are fetched before any of them is stored
+    int drow[16];
+    u32x2 res[16];
+    if (EPI == EPI_RESIDUAL_BF16) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int m = mrow0 + i * 32 + 8 * g;
+        if (a.dst_row) {
+          if (m + 3 < a.M) {
+            const i32x4 d = *reinterpret_cast<const i32x4*>(a.dst_row + m);
+            drow[4 * g] = d[0]; drow[4 * g + 1] = d[1]; drow[4 * g + 2] = d[2]; drow[4 * g + 3] = d[3];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) drow[4 * g + e] = (m + e < a.M) ? a.dst_row[m + e] : -1;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) drow[4 * g + e] = (m + e < a.M) ? m + e : -1;
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const u32x2 z = {0u, 0u};
+        res[r] = z;
+        if (drow[r] >= 0)
+          res[r] = *reinterpret_cast<const u32x2*>(a.residual + (int64_t)drow[r] * a.ld_res + nc);
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int m = mrow0 + i * 32 + 8 * (r >> 2) + (r & 3);
-      if (m < a.M) {
+      const int orow = (EPI == EPI_RESIDUAL_BF16) ? drow[r] : (m < a.M ? m : -1);
+      if (orow >= 0) {
         const float s = sxv[i][r >> 2][r & 3];
         float y[4];
 #pragma unroll
@@ -225,15 +274,29 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
           t = t * swv[j];
           y[j] = t + bv4[j];
         }
-        const u32x2 o = {pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3])};
-        *reinterpret_cast<u32x2*>(reinterpret_cast<unsigned short*>(a.out) + (int64_t)m * a.ldo + nc) = o;
+        u32x2 o = {pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3])};
+        if (EPI == EPI_GELU_BF16) {
+          // activation of the bf16-rounded Linear output, as a separate GELU would see it
+          o[0] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[0])), gelu_erf(bf16_hi_to_f32(o[0])));
+          o[1] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[1])), gelu_erf(bf16_hi_to_f32(o[1])));
+        }
+        if (EPI == EPI_RESIDUAL_BF16) {
+          // bf16 add of the bf16-rounded Linear output and the residual stream
+          o[0] = pack_bf16x2(bf16_lo_to_f32(o[0]) + bf16_lo_to_f32(res[r][0]),
+                             bf16_hi_to_f32(o[0]) + bf16_hi_to_f32(res[r][0]));
+          o[1] = pack_bf16x2(bf16_lo_to_f32(o[1]) + bf16_lo_to_f32(res[r][1]),
+                             bf16_hi_to_f32(o[1]) + bf16_hi_to_f32(res[r][1]));
+        }
+        *reinterpret_cast<u32x2*>(reinterpret_cast<unsigned short*>(a.out) + (int64_t)orow * a.ldo + nc) = o;
       }
     }
+  }
 }
 
 static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t* wq,
                        const float* sw, const float* bias, void* out, int64_t ldo, int64_t M,
-                       int N, int K, hipStream_t stream) {
+                       int N, int K, hipStream_t stream, const void* residual = nullptr,
+                       int64_t ld_res = 0, const int32_t* dst_row = nullptr) {
   SF_REQUIRE(xq && wq && out, "gemm_i8: null pointer");
   SF_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_i8: bad shape M=%lld N=%d K=%d", (long long)M, N, K);
   SF_REQUIRE(M < (1ll << 31) - 256, "gemm_i8: M=%lld too large", (long long)M);
@@ -254,6 +317,14 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   GemmArgs a;
   a.x = xq; a.w = wq; a.out = out; a.sx = sx; a.sw = sw; a.bias = bias;
   a.ldo = ldo; a.M = (int)M; a.N = N; a.K = K;
+  a.residual = reinterpret_cast<const unsigned short*>(residual);
+  a.ld_res = ld_res; a.dst_row = dst_row;
+  if (epi == EPI_RESIDUAL_BF16) {
+    SF_REQUIRE(residual && (reinterpret_cast<uintptr_t>(residual) & 7u) == 0 && ld_res >= N &&
+                   ld_res % 4 == 0,
+               "gemm_i8: residual must be non-null with 8-byte aligned rows");
+    SF_REQUIRE(!dst_row || aligned16(dst_row), "gemm_i8: dst_row must be 16-byte aligned");
+  }
   const char* force = getenv("SAMFAST_GEMM_TM");  // tuning aid: 2 or 4
   const int tm = force ? atoi(force) : 2;
   const int bm = 64 * tm;
@@ -262,13 +333,18 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   const int64_t total = (int64_t)a.tiles_m * a.tiles_n;
   SF_REQUIRE(total < (1ll << 30), "gemm_i8: too many tiles");
   const unsigned int grid = (unsigned int)(((total + 7) / 8) * 8);
-  if (epi == EPI_I32) {
-    if (tm == 4) hipLaunchKernelGGL((gemm_i8_kernel<EPI_I32, 4>), dim3(grid), dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL((gemm_i8_kernel<EPI_I32, 2>), dim3(grid), dim3(256), 0, stream, a);
-  } else {
-    if (tm == 4) hipLaunchKernelGGL((gemm_i8_kernel<EPI_SCALE_BIAS_BF16, 4>), dim3(grid), dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL((gemm_i8_kernel<EPI_SCALE_BIAS_BF16, 2>), dim3(grid), dim3(256), 0, stream, a);
+#define SF_GEMM_LAUNCH(E)                                                                          \
+  do {                                                                                             \
+    if (tm == 4) hipLaunchKernelGGL((gemm_i8_kernel<E, 4>), dim3(grid), dim3(256), 0, stream, a);  \
+    else hipLaunchKernelGGL((gemm_i8_kernel<E, 2>), dim3(grid), dim3(256), 0, stream, a);          \
+  } while (0)
+  switch (epi) {
+    case EPI_I32: SF_GEMM_LAUNCH(EPI_I32); break;
+    case EPI_SCALE_BIAS_BF16: SF_GEMM_LAUNCH(EPI_SCALE_BIAS_BF16); break;
+    case EPI_GELU_BF16: SF_GEMM_LAUNCH(EPI_GELU_BF16); break;
+    default: SF_GEMM_LAUNCH(EPI_RESIDUAL_BF16); break;
   }
+#undef SF_GEMM_LAUNCH
   return check_launch("gemm_i8_kernel");
 }
 
@@ -289,4 +365,27 @@ extern "C" int samfast_gemm_i8_scale_bias(const int8_t* xq, const float* sx, con
   }
   return samfast::gemm_common(samfast::EPI_SCALE_BIAS_BF16, xq, sx, wq, sw, bias, y, ldy, M, N, K,
                               reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int samfast_gemm_i8_fused(const int8_t* xq, const float* sx, const int8_t* wq,
+                                     const float* sw, const float* bias, void* y, int64_t ldy,
+                                     int64_t M, int N, int K, int dtype, int epilogue,
+                                     const void* residual, int64_t ld_res, const int32_t* dst_row,
+                                     void* stream) {
+  using namespace samfast;
+  if (dtype != SAMFAST_BF16) {
+    set_error("gemm_i8_fused: only bf16 output");
+    return SAMFAST_E_UNSUPPORTED;
+  }
+  int epi;
+  switch (epilogue) {
+    case SAMFAST_EPILOGUE_NONE: epi = EPI_SCALE_BIAS_BF16; break;
+    case SAMFAST_EPILOGUE_GELU: epi = EPI_GELU_BF16; break;
+    case SAMFAST_EPILOGUE_RESIDUAL: epi = EPI_RESIDUAL_BF16; break;
+    default:
+      set_error("gemm_i8_fused: unknown epilogue %d", epilogue);
+      return SAMFAST_E_INVALID;
+  }
+  return gemm_common(epi, xq, sx, wq, sw, bias, y, ldy, M, N, K,
+                     reinterpret_cast<hipStream_t>(stream), residual, ld_res, dst_row);
 }

@@ -1,9 +1,16 @@
-// Per-row symmetric int8 quantiser (bf16 -> int8 + fp32 scale), HBM-bound.
+// Per-row symmetric int8 quantiser (bf16 -> int8 + fp32 scale), optionally preceded
+// by LayerNorm over the row and a row gather (window partition).  HBM-bound.
 //
-// One wavefront owns one row: the row is read once with 16-byte loads into
-// registers, reduced to its absmax across the 64 lanes, then divided, rounded
-// half-to-even and written back as 8-byte packs of int8.  Algorithmic traffic is
-// 2 bytes read + 1 byte written per element plus 4 bytes of scale per row.
+// One wavefront owns one output row: the source row is read once with 16-byte loads
+// into registers, (normalised,) reduced to its absmax across the 64 lanes, then
+// scaled, rounded half-to-even and written back as 8-byte packs of int8.
+// Algorithmic traffic: 2 bytes read + 1 byte written per element + 4 bytes of scale.
+//
+// q = rint(x / s) must equal the IEEE division bit for bit.  Most elements take a
+// cheap route: r = x * (1/s) differs from x / s by a few ulp, so rint(r) can only
+// differ when r lies within 1e-4 of a half-integer; only those elements (and their
+// 8-element chunk) are redone with the true division.  |x| <= absmax makes
+// |x / s| <= 127 by construction, so no clamp is needed.
 #include "samfast_internal.hpp"
 
 // every fp32 step below is rounded on its own (no fused multiply-add), so results
@@ -14,67 +21,186 @@ namespace samfast {
 
 constexpr int kQuantWavesPerBlock = 4;
 
-template <int NCH>  // 16-byte chunks per lane: covers K <= NCH * 512
-__global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_kernel(
-    const unsigned short* __restrict__ x, int64_t ldx, int8_t* __restrict__ xq,
-    float* __restrict__ sx, int64_t M, int K) {
+struct QuantArgs {
+  const unsigned short* x;
+  int64_t ldx;
+  const unsigned short* gamma;  // LN only
+  const unsigned short* beta;   // LN only
+  const int32_t* src_row;       // LN only: source row per output row, -1 = all-zero row; may be null
+  int8_t* xq;
+  float* sx;
+  int64_t M;
+  int K;
+  float eps;
+};
+
+SF_DEVICE float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+SF_DEVICE float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// 8 values -> 8 int8 codes packed in 8 bytes
+SF_DEVICE u32x2 quantize8(const float (&v)[8], float scale, float inv_scale) {
+  float r[8];
+  bool near_tie = false;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    r[e] = v[e] * inv_scale;
+    const float frac = r[e] - floorf(r[e]);
+    near_tie |= fabsf(frac - 0.5f) < 1e-4f;
+  }
+  if (near_tie) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = v[e] / scale;  // IEEE division
+  }
+  unsigned int p[2] = {0u, 0u};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int q = (int)rintf(r[e]);
+    p[e >> 2] |= ((unsigned int)(q & 0xff)) << (8 * (e & 3));
+  }
+  const u32x2 o = {p[0], p[1]};
+  return o;
+}
+
+template <int NCH, bool LN>  // 16-byte chunks per lane: covers K <= NCH * 512
+__global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_kernel(QuantArgs a) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * kQuantWavesPerBlock + (threadIdx.x >> 6);
-  if (row >= M) return;  // whole wavefront leaves together
-  const int nchunk = K >> 3;
-  const u32x4* src = reinterpret_cast<const u32x4*>(x + row * ldx);
+  if (row >= a.M) return;  // whole wavefront leaves together
+  const int nchunk = a.K >> 3;
+  u32x2* dst = reinterpret_cast<u32x2*>(a.xq + row * (int64_t)a.K);
+
+  int64_t srow = row;
+  if (LN && a.src_row) {
+    srow = a.src_row[row];
+    if (srow < 0) {  // a padding token: LayerNorm output replaced by zeros
+      const u32x2 z = {0u, 0u};
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int c = lane + i * 64;
+        if (c < nchunk) dst[c] = z;
+      }
+      if (lane == 0) a.sx[row] = 1e-5f / 127.0f;
+      return;
+    }
+  }
+  const u32x4* src = reinterpret_cast<const u32x4*>(a.x + srow * a.ldx);
 
   u32x4 buf[NCH];
-  float amax = 0.f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = lane + i * 64;
     u32x4 w = {0u, 0u, 0u, 0u};
     if (c < nchunk) w = src[c];
     buf[i] = w;
+  }
+
+  if (LN) {
+    // two-pass mean / biased variance over the K real elements, fp32
+    float s1 = 0.f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      amax = fmaxf(amax, fabsf(bf16_lo_to_f32(w[j])));
-      amax = fmaxf(amax, fabsf(bf16_hi_to_f32(w[j])));
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s1 += bf16_lo_to_f32(buf[i][j]) + bf16_hi_to_f32(buf[i][j]);
+    const float mean = wave_sum(s1) / (float)a.K;
+    float s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      if (lane + i * 64 < nchunk) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float d0 = bf16_lo_to_f32(buf[i][j]) - mean, d1 = bf16_hi_to_f32(buf[i][j]) - mean;
+          s2 += d0 * d0 + d1 * d1;
+        }
+      }
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(s2) / (float)a.K + a.eps);
+    const u32x4* g4 = reinterpret_cast<const u32x4*>(a.gamma);
+    const u32x4* b4 = reinterpret_cast<const u32x4*>(a.beta);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = lane + i * 64;
+      if (c < nchunk) {
+        const u32x4 g = g4[c], b = b4[c];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float y0 = (bf16_lo_to_f32(buf[i][j]) - mean) * rstd * bf16_lo_to_f32(g[j]) + bf16_lo_to_f32(b[j]);
+          const float y1 = (bf16_hi_to_f32(buf[i][j]) - mean) * rstd * bf16_hi_to_f32(g[j]) + bf16_hi_to_f32(b[j]);
+          buf[i][j] = pack_bf16x2(y0, y1);  // the bf16 value a separate LayerNorm would have stored
+        }
+      }
     }
   }
+
+  float amax = 0.f;
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+  for (int i = 0; i < NCH; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      amax = fmaxf(amax, fabsf(bf16_lo_to_f32(buf[i][j])));
+      amax = fmaxf(amax, fabsf(bf16_hi_to_f32(buf[i][j])));
+    }
+  amax = wave_max(amax);
 
   const float scale = fmaxf(amax, 1e-5f) / 127.0f;
-  if (lane == 0) sx[row] = scale;
+  const float inv_scale = 1.0f / scale;
+  if (lane == 0) a.sx[row] = scale;
 
-  u32x2* dst = reinterpret_cast<u32x2*>(xq + row * (int64_t)K);
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = lane + i * 64;
     if (c < nchunk) {
-      unsigned int packed[2] = {0u, 0u};
+      float v[8];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float lo = bf16_lo_to_f32(buf[i][j]);
-        const float hi = bf16_hi_to_f32(buf[i][j]);
-        // IEEE division, then round half to even, then clamp
-        const int qlo = (int)fminf(fmaxf(rintf(lo / scale), -127.f), 127.f);
-        const int qhi = (int)fminf(fmaxf(rintf(hi / scale), -127.f), 127.f);
-        const int e = 2 * j;  // element index inside the chunk
-        packed[e >> 2] |= ((unsigned int)(qlo & 0xff)) << (8 * (e & 3));
-        packed[(e + 1) >> 2] |= ((unsigned int)(qhi & 0xff)) << (8 * ((e + 1) & 3));
+        v[2 * j] = bf16_lo_to_f32(buf[i][j]);
+        v[2 * j + 1] = bf16_hi_to_f32(buf[i][j]);
       }
-      u32x2 o = {packed[0], packed[1]};
-      dst[c] = o;
+      dst[c] = quantize8(v, scale, inv_scale);
     }
   }
 }
 
-template <int NCH>
-static int launch_quant(const void* x, int64_t ldx, int8_t* xq, float* sx, int64_t M, int K,
-                        hipStream_t stream) {
-  const int64_t blocks = (M + kQuantWavesPerBlock - 1) / kQuantWavesPerBlock;
-  hipLaunchKernelGGL(quant_rowwise_bf16_kernel<NCH>, dim3((unsigned int)blocks),
-                     dim3(64 * kQuantWavesPerBlock), 0, stream,
-                     reinterpret_cast<const unsigned short*>(x), ldx, xq, sx, M, K);
+template <int NCH, bool LN>
+static int launch_quant(const QuantArgs& a, hipStream_t stream) {
+  const int64_t blocks = (a.M + kQuantWavesPerBlock - 1) / kQuantWavesPerBlock;
+  hipLaunchKernelGGL((quant_rowwise_bf16_kernel<NCH, LN>), dim3((unsigned int)blocks),
+                     dim3(64 * kQuantWavesPerBlock), 0, stream, a);
   return check_launch("quant_rowwise_bf16_kernel");
+}
+
+template <bool LN>
+static int dispatch_quant(const QuantArgs& a, hipStream_t s) {
+  const int need = (a.K / 8 + 63) / 64;
+  if (need <= 2) return launch_quant<2, LN>(a, s);
+  if (need <= 3) return launch_quant<3, LN>(a, s);
+  if (need <= 4) return launch_quant<4, LN>(a, s);
+  if (need <= 6) return launch_quant<6, LN>(a, s);
+  if (need <= 8) return launch_quant<8, LN>(a, s);
+  if (need <= 10) return launch_quant<10, LN>(a, s);
+  if (need <= 12) return launch_quant<12, LN>(a, s);
+  return launch_quant<16, LN>(a, s);
+}
+
+static int check_common(const char* who, const void* x, int64_t ldx, const int8_t* xq, const float* sx,
+                        int64_t M, int K, int dtype) {
+  SF_REQUIRE(x && xq && sx, "%s: null pointer", who);
+  SF_REQUIRE(M >= 0 && K > 0, "%s: bad shape M=%lld K=%d", who, (long long)M, K);
+  if (dtype != SAMFAST_BF16) SF_FAIL(SAMFAST_E_UNSUPPORTED, "%s: only bf16 input", who);
+  SF_REQUIRE(K % 8 == 0 && K <= 8192, "%s: K=%d must be a multiple of 8, <= 8192", who, K);
+  SF_REQUIRE(ldx >= K && ldx % 8 == 0, "%s: ldx=%lld must be >= K and a multiple of 8", who,
+             (long long)ldx);
+  SF_REQUIRE(aligned16(x) && (reinterpret_cast<uintptr_t>(xq) & 7u) == 0,
+             "%s: x must be 16-byte and xq 8-byte aligned", who);
+  SF_REQUIRE((M + 3) / 4 < (1ll << 31), "%s: M too large", who);
+  return SAMFAST_OK;
 }
 
 }  // namespace samfast
@@ -82,24 +208,31 @@ static int launch_quant(const void* x, int64_t ldx, int8_t* xq, float* sx, int64
 extern "C" int samfast_quant_rowwise_i8(const void* x, int64_t ldx, int8_t* xq, float* sx,
                                         int64_t M, int K, int dtype, void* stream) {
   using namespace samfast;
-  SF_REQUIRE(x && xq && sx, "quant_rowwise: null pointer");
-  SF_REQUIRE(M >= 0 && K > 0, "quant_rowwise: bad shape M=%lld K=%d", (long long)M, K);
-  if (dtype != SAMFAST_BF16) SF_FAIL(SAMFAST_E_UNSUPPORTED, "quant_rowwise: only bf16 input");
-  SF_REQUIRE(K % 8 == 0 && K <= 8192, "quant_rowwise: K=%d must be a multiple of 8, <= 8192", K);
-  SF_REQUIRE(ldx >= K && ldx % 8 == 0, "quant_rowwise: ldx=%lld must be >= K and a multiple of 8",
-             (long long)ldx);
-  SF_REQUIRE(aligned16(x) && (reinterpret_cast<uintptr_t>(xq) & 7u) == 0,
-             "quant_rowwise: x must be 16-byte and xq 8-byte aligned");
-  SF_REQUIRE((M + 3) / 4 < (1ll << 31), "quant_rowwise: M too large");
+  const int rc = check_common("quant_rowwise", x, ldx, xq, sx, M, K, dtype);
+  if (rc != SAMFAST_OK) return rc;
   if (M == 0) return SAMFAST_OK;
-  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  const int need = (K / 8 + 63) / 64;
-  if (need <= 2) return launch_quant<2>(x, ldx, xq, sx, M, K, s);
-  if (need <= 3) return launch_quant<3>(x, ldx, xq, sx, M, K, s);
-  if (need <= 4) return launch_quant<4>(x, ldx, xq, sx, M, K, s);
-  if (need <= 6) return launch_quant<6>(x, ldx, xq, sx, M, K, s);
-  if (need <= 8) return launch_quant<8>(x, ldx, xq, sx, M, K, s);
-  if (need <= 10) return launch_quant<10>(x, ldx, xq, sx, M, K, s);
-  if (need <= 12) return launch_quant<12>(x, ldx, xq, sx, M, K, s);
-  return launch_quant<16>(x, ldx, xq, sx, M, K, s);
+  QuantArgs a = {};
+  a.x = reinterpret_cast<const unsigned short*>(x);
+  a.ldx = ldx; a.xq = xq; a.sx = sx; a.M = M; a.K = K;
+  return dispatch_quant<false>(a, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int samfast_layernorm_quant_i8(const void* x, int64_t ldx, const void* gamma,
+                                          const void* beta, float eps, const int32_t* src_row,
+                                          int8_t* xq, float* sx, int64_t M, int K, int dtype,
+                                          void* stream) {
+  using namespace samfast;
+  const int rc = check_common("layernorm_quant", x, ldx, xq, sx, M, K, dtype);
+  if (rc != SAMFAST_OK) return rc;
+  SF_REQUIRE(gamma && beta && aligned16(gamma) && aligned16(beta),
+             "layernorm_quant: gamma / beta must be non-null and 16-byte aligned");
+  SF_REQUIRE(eps > 0.f, "layernorm_quant: eps must be positive");
+  if (M == 0) return SAMFAST_OK;
+  QuantArgs a = {};
+  a.x = reinterpret_cast<const unsigned short*>(x);
+  a.ldx = ldx; a.xq = xq; a.sx = sx; a.M = M; a.K = K;
+  a.gamma = reinterpret_cast<const unsigned short*>(gamma);
+  a.beta = reinterpret_cast<const unsigned short*>(beta);
+  a.src_row = src_row; a.eps = eps;
+  return dispatch_quant<true>(a, reinterpret_cast<hipStream_t>(stream));
 }

@@ -29,7 +29,14 @@ _SIGNATURES = {
     "samfast_gemm_i8_i32": (_i32, [_ptr, _ptr, _ptr, _i64, _i32, _i32, _ptr]),
     "samfast_gemm_i8_scale_bias": (
         _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _ptr]),
+    "samfast_layernorm_quant_i8": (
+        _i32, [_ptr, _i64, _ptr, _ptr, _f32, _ptr, _ptr, _ptr, _i64, _i32, _i32, _ptr]),
+    "samfast_gemm_i8_fused": (
+        _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _i32,
+               _ptr, _i64, _ptr, _ptr]),
 }
+
+EPILOGUE_NONE, EPILOGUE_GELU, EPILOGUE_RESIDUAL = 0, 1, 2
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

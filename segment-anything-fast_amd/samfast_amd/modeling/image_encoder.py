@@ -13,18 +13,27 @@ rel_pos_h / rel_pos_w, and the result is written token-major, so the head
 split/merge copies (:228-230, :249) and the bias tensors (:234-242) never exist.
 Any other input (CPU, fp32, shapes the kernels do not cover) follows the
 reference's own composition through flash_4._attention_rel_h_rel_w.
+
+When, in addition, the four Linears of a Block have been swapped for
+quant.Int8DynamicLinear, Block.forward (:167-183) runs as nine kernel launches with
+no eager glue: LayerNorm + window partition + quantise, qkv GEMM, attention,
+quantise, proj GEMM + window unpartition + residual, LayerNorm + quantise, lin1 GEMM
++ GELU, quantise, lin2 GEMM + residual.  SAMFAST_FUSED_BLOCK=0 keeps the
+module-by-module composition instead.
 """
 
+import os
 from typing import Optional, Tuple, Type
 
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .. import ops
-from .. import flash_4
+from .. import _lib, flash_4, ops
 from ..flash_4 import _attention_rel_h_rel_w
 from .common import LayerNorm2d, MLPBlock
+
+FUSED_BLOCK = bool(int(os.environ.get("SAMFAST_FUSED_BLOCK", 1)))
 
 
 class ImageEncoderViT(nn.Module):
@@ -108,7 +117,63 @@ class Block(nn.Module):
         self.mlp = MLPBlock(embedding_dim=dim, mlp_dim=int(dim * mlp_ratio), act=act_layer)
         self.window_size = window_size
 
+    def _int8_fused_ok(self, x: torch.Tensor) -> bool:
+        from ..quant import Int8DynamicLinear
+        attn, mlp = self.attn, self.mlp
+        if not (FUSED_BLOCK and flash_4.USE_CUSTOM_KERNEL and x.is_cuda
+                and x.dtype == torch.bfloat16 and x.dim() == 4 and attn.use_rel_pos):
+            return False
+        if not all(isinstance(m, Int8DynamicLinear) for m in (attn.qkv, attn.proj, mlp.lin1, mlp.lin2)):
+            return False
+        if not (isinstance(self.norm1, nn.LayerNorm) and isinstance(self.norm2, nn.LayerNorm)
+                and self.norm1.elementwise_affine and self.norm2.elementwise_affine
+                and self.norm1.bias is not None and self.norm2.bias is not None
+                and self.norm1.weight.dtype == torch.bfloat16
+                and isinstance(mlp.act, nn.GELU) and getattr(mlp.act, "approximate", "none") == "none"):
+            return False
+        B, H, W, C = x.shape
+        g = self.window_size if self.window_size > 0 else None
+        gh, gw = (g, g) if g else (H, W)
+        return (attn.rel_pos_h.shape[0] == 2 * gh - 1 and attn.rel_pos_w.shape[0] == 2 * gw - 1
+                and ops.attn_supported(gh * gw, (gh, gw), C // attn.num_heads, x.dtype))
+
+    def _forward_int8_fused(self, x: torch.Tensor) -> torch.Tensor:
+        """image_encoder.py:167-183 with every step on the HIP kernels."""
+        B, H, W, C = x.shape
+        attn, mlp = self.attn, self.mlp
+        nH = attn.num_heads
+        hd = C // nH
+        tokens = x.contiguous().view(B * H * W, C)
+        if self.window_size > 0:
+            ws = self.window_size
+            row_map, _ = ops.window_row_maps(B, H, W, ws, x.device)
+            gh = gw = ws
+        else:
+            row_map = None
+            gh, gw = H, W
+        N = gh * gw
+        # norm1 (+ window partition with zero padding) + qkv's activation quantiser
+        xq, sx = ops.layernorm_quant(tokens, self.norm1.weight, self.norm1.bias, self.norm1.eps, row_map)
+        Bw = xq.shape[0] // N
+        qkv = ops.gemm_i8_fused(xq, sx, attn.qkv.wq, attn.qkv.sw, attn.qkv.bias_f32, _lib.EPILOGUE_NONE)
+        qkv = qkv.view(Bw, N, 3, nH, hd)
+        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        o = ops.attn_relpos(q, k, v, attn.rel_pos_h, attn.rel_pos_w, (gh, gw), attn.scale)
+        oq, so = ops.quant_rowwise(o.permute(0, 2, 1, 3).reshape(Bw * N, C))
+        # proj + window unpartition + `shortcut + x`
+        tokens = ops.gemm_i8_fused(oq, so, attn.proj.wq, attn.proj.sw, attn.proj.bias_f32,
+                                   _lib.EPILOGUE_RESIDUAL, residual=tokens, dst_row=row_map)
+        # norm2 + lin1's quantiser, lin1 + GELU, lin2's quantiser, lin2 + `x + mlp(...)`
+        hq, sh = ops.layernorm_quant(tokens, self.norm2.weight, self.norm2.bias, self.norm2.eps)
+        h = ops.gemm_i8_fused(hq, sh, mlp.lin1.wq, mlp.lin1.sw, mlp.lin1.bias_f32, _lib.EPILOGUE_GELU)
+        gq, sg = ops.quant_rowwise(h)
+        tokens = ops.gemm_i8_fused(gq, sg, mlp.lin2.wq, mlp.lin2.sw, mlp.lin2.bias_f32,
+                                   _lib.EPILOGUE_RESIDUAL, residual=tokens, out=tokens)
+        return tokens.view(B, H, W, C)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self._int8_fused_ok(x):
+            return self._forward_int8_fused(x)
         shortcut = x
         x = self.norm1(x)
         if self.window_size > 0:

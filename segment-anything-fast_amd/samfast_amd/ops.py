@@ -215,3 +215,97 @@ def gemm_i8_scale_bias(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw:
             M, N, K, _lib.SAMFAST_BF16, _stream()))
     _lib.check(code, "gemm_i8_scale_bias")
     return out
+
+
+def layernorm_quant(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, eps: float,
+                    src_row: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """LayerNorm over the last axis of x (R, K) bf16, optional row gather (src_row int32 (M,),
+    -1 = zero row), then the per-row int8 quantiser.  Returns (int8 (M, K), fp32 (M,))."""
+    _require_gpu(x, gamma, beta, src_row)
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise RuntimeError("samfast: layernorm_quant needs a 2-D tensor with contiguous rows")
+    K = x.shape[1]
+    M = x.shape[0] if src_row is None else src_row.numel()
+    if gamma.dtype != x.dtype or beta.dtype != x.dtype or gamma.numel() != K or beta.numel() != K:
+        raise RuntimeError("samfast: gamma / beta must match x in dtype and length K")
+    if src_row is not None and (src_row.dtype != torch.int32 or not src_row.is_contiguous()):
+        raise RuntimeError("samfast: src_row must be a contiguous int32 tensor")
+    xq = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    sx = torch.empty((M,), dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    code = _timed(
+        "layernorm_quant", 2.0 * min(M, x.shape[0]) * K + 1.0 * M * K + 4.0 * M, "byte",
+        lambda: lib.samfast_layernorm_quant_i8(
+            x.data_ptr(), x.stride(0), gamma.contiguous().data_ptr(), beta.contiguous().data_ptr(),
+            float(eps), src_row.data_ptr() if src_row is not None else None,
+            xq.data_ptr(), sx.data_ptr(), M, K, _dtype_code(x), _stream()))
+    _lib.check(code, "layernorm_quant_i8")
+    return xq, sx
+
+
+def gemm_i8_fused(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor,
+                  bias: Optional[torch.Tensor], epilogue: int,
+                  residual: Optional[torch.Tensor] = None, dst_row: Optional[torch.Tensor] = None,
+                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """gemm_i8_scale_bias with a fused tail (see include/samfast.h):
+    _lib.EPILOGUE_GELU, or _lib.EPILOGUE_RESIDUAL with `residual` (rows_out, N) bf16 and an
+    optional int32 row scatter `dst_row` (M,), -1 = dropped.  For RESIDUAL the output has the
+    shape of `residual` (and may alias it via `out=residual`)."""
+    _require_gpu(xq, sx, wq, sw, bias, residual, dst_row)
+    if not (xq.is_contiguous() and wq.is_contiguous()) or xq.shape[1] != wq.shape[1]:
+        raise RuntimeError("samfast: gemm_i8_fused needs contiguous (M, K) and (N, K)")
+    M, K = xq.shape
+    N = wq.shape[0]
+    if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != M or sw.numel() != N:
+        raise RuntimeError("samfast: scales must be fp32 of length M and N")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N):
+        raise RuntimeError("samfast: bias must be fp32 of length N")
+    if epilogue == _lib.EPILOGUE_RESIDUAL:
+        if residual is None or residual.dim() != 2 or residual.shape[1] != N or residual.stride(1) != 1 \
+                or residual.dtype != torch.bfloat16:
+            raise RuntimeError("samfast: residual must be a bf16 (rows, N) tensor")
+        if dst_row is None and residual.shape[0] != M:
+            raise RuntimeError("samfast: residual rows must equal M without a row map")
+        if dst_row is not None and (dst_row.dtype != torch.int32 or dst_row.numel() != M
+                                    or not dst_row.is_contiguous()):
+            raise RuntimeError("samfast: dst_row must be a contiguous int32 tensor of length M")
+        if out is None:
+            out = torch.empty_like(residual)
+    elif out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=xq.device)
+    lib = _lib.load()
+    name = {_lib.EPILOGUE_NONE: "gemm_i8_scale_bias", _lib.EPILOGUE_GELU: "gemm_i8_gelu",
+            _lib.EPILOGUE_RESIDUAL: "gemm_i8_residual"}.get(epilogue, "gemm_i8_fused")
+    code = _timed(
+        name, 2.0 * M * N * K, "op",
+        lambda: lib.samfast_gemm_i8_fused(
+            xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
+            bias.data_ptr() if bias is not None else None, out.data_ptr(), out.stride(0),
+            M, N, K, _lib.SAMFAST_BF16, int(epilogue),
+            residual.data_ptr() if residual is not None else None,
+            residual.stride(0) if residual is not None else 0,
+            dst_row.data_ptr() if dst_row is not None else None, _stream()))
+    _lib.check(code, "gemm_i8_fused")
+    return out
+
+
+_window_maps = {}
+
+
+def window_row_maps(B: int, H: int, W: int, window: int, device) -> Tuple[torch.Tensor, Tuple[int, int]]:
+    """int32 map for window_partition on (B, H, W) tokens: entry r of the window-ordered,
+    zero-padded token list holds the flat index of its source token, or -1 for a padding
+    position.  The same tensor is the scatter map of window_unpartition.  Cached."""
+    key = (B, H, W, window, str(device))
+    hit = _window_maps.get(key)
+    if hit is not None:
+        return hit
+    Hp = H + (-H) % window
+    Wp = W + (-W) % window
+    idx = torch.arange(B * H * W, dtype=torch.int32).view(B, H, W)
+    padded = torch.full((B, Hp, Wp), -1, dtype=torch.int32)
+    padded[:, :H, :W] = idx
+    wins = padded.view(B, Hp // window, window, Wp // window, window).permute(0, 1, 3, 2, 4)
+    res = (wins.reshape(-1).contiguous().to(device), (Hp, Wp))
+    _window_maps[key] = res
+    return res

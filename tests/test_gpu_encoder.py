@@ -104,3 +104,37 @@ def test_predictor_set_torch_image():
     pred.set_torch_image(img, (1024, 768))
     f = pred.get_image_embedding()
     assert f.shape == (1, 256, 64, 64) and f.dtype == torch.bfloat16 and torch.isfinite(f.float()).all()
+
+
+def test_fused_block_equals_module_composition():
+    """Block.forward as nine fused launches against the same block run module by module
+    (LayerNorm, window partition, residual adds and GELU in PyTorch-ROCm), windowed and global."""
+    from samfast_amd import apply_dynamic_quant
+    from samfast_amd.modeling import Block
+    from samfast_amd.modeling import image_encoder as ie
+    for ws in (14, 0):
+        torch.manual_seed(5)
+        blk = Block(1280, 16, use_rel_pos=True, window_size=ws, input_size=(64, 64),
+                    norm_layer=partial(torch.nn.LayerNorm, eps=1e-6))
+        with torch.no_grad():
+            blk.attn.rel_pos_h.normal_(0, 0.02)
+            blk.attn.rel_pos_w.normal_(0, 0.02)
+            blk.norm1.weight.normal_(1, 0.1)
+            blk.norm1.bias.normal_(0, 0.1)
+        blk = blk.eval().to(torch.bfloat16).cuda()
+        apply_dynamic_quant(blk)
+        x = torch.randn(2, 64, 64, 1280, device="cuda").to(torch.bfloat16)
+        with torch.no_grad():
+            assert blk._int8_fused_ok(x)
+            fused = blk(x)
+            ie.FUSED_BLOCK = False
+            try:
+                assert not blk._int8_fused_ok(x)
+                plain = blk(x)
+            finally:
+                ie.FUSED_BLOCK = True
+        d = (fused.float() - plain.float()).abs()
+        c = _cos(fused, plain)
+        print(f"fused block ws={ws}: cosine {c:.6f} max-abs {d.max().item():.4f} mean-abs {d.mean().item():.5f}",
+              flush=True)
+        assert c >= 0.9999 and d.mean().item() <= 2e-3

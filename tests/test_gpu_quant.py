@@ -106,3 +106,89 @@ def test_module_swap_forward():
     out = mlp.cuda()(x.cuda())
     d = (out.float().cpu() - ref.float()).abs().max().item()
     assert d <= 2e-2, d  # GELU on the GPU in bf16 vs fp32 on the CPU: not bit-exact
+
+
+def _oracle_ln_quant(x, gamma, beta, eps, src_row=None):
+    y = torch.nn.functional.layer_norm(x.float(), (x.shape[1],), gamma.float(), beta.float(), eps)
+    y = y.to(torch.bfloat16)
+    if src_row is not None:
+        src = src_row.long()
+        out = torch.zeros((src.numel(), x.shape[1]), dtype=torch.bfloat16)
+        out[src >= 0] = y[src[src >= 0]]
+        y = out
+    return orq.quantize_rows_absmax(y)
+
+
+@pytest.mark.parametrize("R,K", [(64, 768), (300, 1280), (50, 1024)])
+def test_layernorm_quant_vs_oracle(R, K):
+    """LayerNorm is floating point (reduction order differs from the CPU), so codes may
+    differ by one step where the normalised value sits on a rounding boundary:
+    bar = at most 1 code step anywhere, >= 99.5 % identical, scales within 1 %."""
+    from samfast_amd import ops
+    g = torch.Generator().manual_seed(R + K)
+    x = (torch.randn(R, K, generator=g) * 2 + 0.3).to(torch.bfloat16)
+    gamma = (1 + 0.1 * torch.randn(K, generator=g)).to(torch.bfloat16)
+    beta = (0.1 * torch.randn(K, generator=g)).to(torch.bfloat16)
+    q_ref, s_ref = _oracle_ln_quant(x, gamma, beta, 1e-6)
+    q, s = ops.layernorm_quant(x.cuda(), gamma.cuda(), beta.cuda(), 1e-6)
+    q, s = q.cpu().numpy().astype(np.int32), s.cpu().numpy()
+    assert np.abs(q - q_ref.astype(np.int32)).max() <= 1
+    assert (q == q_ref).mean() >= 0.995
+    assert np.allclose(s, s_ref, rtol=1e-2)
+
+
+def test_layernorm_quant_window_gather():
+    """Row map of window_partition: 8x8 tokens, window 3 -> 9x9 padded, 9 windows per image."""
+    from samfast_amd import ops
+    from oracle import relpos_attention as ora
+    B, H, W, K, ws = 2, 8, 8, 256, 3
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(B, H, W, K, generator=g).to(torch.bfloat16)
+    gamma, beta = torch.ones(K, dtype=torch.bfloat16), torch.zeros(K, dtype=torch.bfloat16)
+    row_map, (Hp, Wp) = ops.window_row_maps(B, H, W, ws, "cuda")
+    assert (Hp, Wp) == (9, 9) and row_map.numel() == B * 81
+    # the map is exactly the oracle's window_partition applied to token indices
+    idx = torch.arange(B * H * W, dtype=torch.float32).view(B, H, W, 1) + 1
+    wins, _ = ora.window_partition(idx, ws)
+    assert torch.equal(wins.reshape(-1).to(torch.int32) - 1, row_map.cpu())
+    q_ref, s_ref = _oracle_ln_quant(x.reshape(-1, K), gamma, beta, 1e-6, row_map.cpu())
+    q, s = ops.layernorm_quant(x.cuda().reshape(-1, K), gamma.cuda(), beta.cuda(), 1e-6, row_map)
+    q, s = q.cpu().numpy().astype(np.int32), s.cpu().numpy()
+    pad = row_map.cpu().numpy() < 0
+    assert pad.sum() == B * (81 - 64)
+    assert np.all(q[pad] == 0) and np.all(s[pad] == np.float32(1e-5) / np.float32(127))
+    assert np.abs(q - q_ref.astype(np.int32)).max() <= 1 and (q == q_ref).mean() >= 0.995
+
+
+def test_gemm_fused_gelu_and_residual():
+    from samfast_amd import _lib, ops
+    from samfast_amd.quant import quantize_weight_per_channel
+    M, N, K = 333, 520, 256
+    x, w, b = linear_inputs(M, K, N, seed=12)
+    wq, sw = quantize_weight_per_channel(w)
+    xq_ref, sx_ref = orq.quantize_rows_absmax(x)
+    lin_ref = orq.scale_bias_epilogue(orq.int8_gemm_i32(xq_ref, wq.numpy()), sx_ref, sw.numpy(), b)
+    xq, sx = ops.quant_rowwise(x.cuda())
+    args = (xq, sx, wq.cuda(), sw.cuda(), b.float().cuda())
+    # GELU of the bf16-rounded linear output: erf approximated to 1.5e-7 -> at most one bf16 step
+    got = ops.gemm_i8_fused(*args, _lib.EPILOGUE_GELU).float().cpu()
+    ref = torch.nn.functional.gelu(lin_ref.float()).to(torch.bfloat16).float()
+    assert (got - ref).abs().max() <= 2 ** -7 * ref.abs().max()
+    assert torch.allclose(got, ref, rtol=2 ** -7, atol=1e-6)
+    assert (got == ref).float().mean() >= 0.99
+    # residual, identity rows: bit-exact (bf16 add of bf16 operands)
+    g = torch.Generator().manual_seed(3)
+    res = torch.randn(M, N, generator=g).to(torch.bfloat16)
+    got = ops.gemm_i8_fused(*args, _lib.EPILOGUE_RESIDUAL, residual=res.cuda()).cpu()
+    ref = (lin_ref.float() + res.float()).to(torch.bfloat16)
+    assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
+    # residual with a scatter map that drops rows and permutes the rest, in place
+    perm = torch.randperm(M, generator=g)
+    dst = torch.full((M,), -1, dtype=torch.int32)
+    keep = perm[:250]
+    dst[keep] = torch.arange(250, dtype=torch.int32)
+    res2 = torch.randn(250, N, generator=g).to(torch.bfloat16)
+    buf = res2.clone().cuda()
+    got = ops.gemm_i8_fused(*args, _lib.EPILOGUE_RESIDUAL, residual=buf, dst_row=dst.cuda(), out=buf).cpu()
+    ref = (lin_ref[keep].float() + res2.float()).to(torch.bfloat16)
+    assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
