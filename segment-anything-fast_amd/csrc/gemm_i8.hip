@@ -11,9 +11,9 @@
 // the other.  K advances 64 bytes per iteration through two LDS stages with
 // global loads running two tiles ahead and the MFMA operand fragments of the next
 // k-step (also across the iteration boundary) read from LDS while the current
-// MFMAs execute; one barrier per iteration, placed between the two k-steps.  LDS rows are padded from 64 to 80
-// bytes so that the 16-byte operand reads of consecutive rows fall in distinct
-// bank groups.
+// MFMAs execute; one barrier per iteration, placed between the two k-steps.  LDS rows
+// are 64 bytes with their four 16-byte chunks XOR-swizzled by the row index, so both
+// the tile writes and the operand reads are free of bank conflicts.
 //
 // W rows are stored in LDS in a permuted order (row n of a wave's 128 columns
 // goes to slot (n%4)*32 + n/4) so that MFMA tile j, lane-column c holds output
@@ -25,6 +25,7 @@
 // their X panels and the W matrix in that XCD's L2.
 #include "samfast_internal.hpp"
 #include <stdlib.h>
+#include <type_traits>
 
 // every fp32 step below is rounded on its own (no fused multiply-add), so results
 // can be reproduced bit for bit on a CPU
@@ -33,7 +34,7 @@
 namespace samfast {
 
 constexpr int GBN = 256, GBK = 64;
-constexpr int GLD = GBK + 16;  // padded LDS row, bytes
+constexpr int GLD = GBK;  // LDS row, bytes (unpadded; chunks are XOR-swizzled instead)
 
 enum { EPI_I32 = 0, EPI_SCALE_BIAS_BF16 = 1, EPI_GELU_BF16 = 2, EPI_RESIDUAL_BF16 = 3 };
 
@@ -68,7 +69,13 @@ SF_DEVICE float gelu_erf(float x) {
   return x * phi;
 }
 
-template <int EPI, int TM>
+// 16-byte chunk c of LDS row r lives at chunk position c ^ lds_swizzle(r).  With it the
+// operand reads (one chunk of 8 / 16 consecutive rows per LDS cycle) and the tile writes
+// (4 chunks of 2 / 4 consecutive rows per cycle) both touch every bank once, whether the
+// LDS cycles through 128 or 256 bytes.
+SF_DEVICE int lds_swizzle(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
+
+template <int EPI, int TM, bool GENERIC>
 __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArgs a) {
   constexpr int GBM = 64 * TM;
   constexpr int GSTAGE = (GBM + GBN) * GLD;
@@ -92,8 +99,8 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
   const int n0 = (int)(in_group / gsz) * GBN;
 
   // ---- global -> LDS staging: 16-byte chunks, TM per thread for X and 4 for W ----
-  const int8_t* gx[TM];
-  const int8_t* gw[4];
+  // (32-bit lane offsets from the uniform matrix bases; M*K and N*K fit in 31 bits)
+  int ox[TM], ow[4];
   int lx[TM], lw[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -101,14 +108,16 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
     const int row = c >> 2, kc = c & 3;
     if (i < TM) {
       const int gm = min(m0 + row, a.M - 1);
-      gx[i] = a.x + (int64_t)gm * a.K + kc * 16;
-      lx[i] = row * GLD + kc * 16;
+      ox[i] = gm * a.K + kc * 16;
+      lx[i] = row * GLD + ((kc ^ lds_swizzle(row)) * 16);
     }
-    const int gn = min(n0 + row, a.N - 1);
-    gw[i] = a.w + (int64_t)gn * a.K + kc * 16;
-    const int within = row & 127;
-    const int slot = (row & 128) + (within & 3) * 32 + (within >> 2);
-    lw[i] = GBM * GLD + slot * GLD + kc * 16;
+    // W: consecutive chunk groups go to consecutive LDS slots (no write bank conflicts);
+    // slot s of a 128-column half holds W row (s % 32) * 4 + s / 32 of that half
+    const int slot = row & 127;
+    const int wrow = (row & 128) + (slot & 31) * 4 + (slot >> 5);
+    const int gn = min(n0 + wrow, a.N - 1);
+    ow[i] = gn * a.K + kc * 16;
+    lw[i] = GBM * GLD + row * GLD + ((kc ^ lds_swizzle(row)) * 16);
   }
 
   i32x16 acc[TM][4];
@@ -126,32 +135,38 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
   //   B. barrier: every wave now holds all of tile kt in registers, so stage kt&1 is
   //      free, and tile kt+1 (written in the previous iteration) is visible;
   //   C. read the fragments of k-step 0 of tile kt+1, write tile kt+2 (fetched from
-  //      global memory two iterations ago) into the freed stage, issue the global
-  //      loads of tile kt+4 - all while the MFMAs of k-step 1 run.
-  i32x4 stg_x[2][TM], stg_w[2][4];  // two tiles in flight from global memory
-  auto global_fetch = [&](int kt, int set) {
+  //      global memory into registers one iteration ago) into the freed stage, issue
+  //      the global loads of tile kt+3 - all while the MFMAs of k-step 1 run.
+  i32x4 stg_x[TM], stg_w[4];
+  auto global_fetch = [&](int kt) {
+    const int8_t* xb = a.x + kt * GBK;  // uniform
+    const int8_t* wb = a.w + kt * GBK;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      if (i < TM) stg_x[set][i] = *reinterpret_cast<const i32x4*>(gx[i] + (int64_t)kt * GBK);
-      stg_w[set][i] = *reinterpret_cast<const i32x4*>(gw[i] + (int64_t)kt * GBK);
+      if (i < TM) stg_x[i] = *reinterpret_cast<const i32x4*>(xb + ox[i]);
+      stg_w[i] = *reinterpret_cast<const i32x4*>(wb + ow[i]);
     }
   };
-  auto lds_store = [&](int stage, int set) {
+  auto lds_store = [&](int stage) {
     unsigned char* dst = lds + stage * GSTAGE;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      if (i < TM) *reinterpret_cast<i32x4*>(dst + lx[i]) = stg_x[set][i];
-      *reinterpret_cast<i32x4*>(dst + lw[i]) = stg_w[set][i];
+      if (i < TM) *reinterpret_cast<i32x4*>(dst + lx[i]) = stg_x[i];
+      *reinterpret_cast<i32x4*>(dst + lw[i]) = stg_w[i];
     }
   };
-  const int a_off = (wm * 32 * TM + lr) * GLD + lh * 16;
-  const int b_off = GBM * GLD + (wn * 128 + lr) * GLD + lh * 16;
+  // fragment of k-step s: chunk 2s + lh of row (tile row base + lr); the swizzle only
+  // depends on lr because every tile row base is a multiple of 32
+  const int frag_chunk = (lh ^ lds_swizzle(lr)) * 16;
+  const int a_off = (wm * 32 * TM + lr) * GLD + frag_chunk;
+  const int b_off = GBM * GLD + (wn * 128 + lr) * GLD + frag_chunk;
   auto load_frags = [&](int stage, int step, i32x4 (&av)[TM], i32x4 (&bv)[4]) {
-    const unsigned char* src = lds + stage * GSTAGE + step * 32;
+    const unsigned char* src = lds + stage * GSTAGE;
+    const int flip = step * 32;  // (2*step + lh) ^ swz == ((lh ^ swz) ^ 2*step) as a chunk index
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      if (i < TM) av[i] = *reinterpret_cast<const i32x4*>(src + a_off + i * 32 * GLD);
-      bv[i] = *reinterpret_cast<const i32x4*>(src + b_off + i * 32 * GLD);
+      if (i < TM) av[i] = *reinterpret_cast<const i32x4*>(src + ((a_off + i * 32 * GLD) ^ flip));
+      bv[i] = *reinterpret_cast<const i32x4*>(src + ((b_off + i * 32 * GLD) ^ flip));
     }
   };
   auto mma = [&](const i32x4 (&av)[TM], const i32x4 (&bv)[4]) {
@@ -163,36 +178,82 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
   };
 
   const int nk = a.K / GBK;
-  global_fetch(0, 0);
-  if (nk > 1) global_fetch(1, 1);
-  lds_store(0, 0);
-  if (nk > 2) global_fetch(2, 0);
-  if (nk > 1) lds_store(1, 1);
-  if (nk > 3) global_fetch(3, 1);
+  global_fetch(0);
+  lds_store(0);
+  if (nk > 1) {
+    global_fetch(1);
+    lds_store(1);
+  }
+  if (nk > 2) global_fetch(2);
   __syncthreads();
 
   i32x4 fa0[TM], fb0[4], fa1[TM], fb1[4];
   load_frags(0, 0, fa0, fb0);
-  // tile kt+2 sits in register set kt&1, tile kt+3 in the other one
-  auto iteration = [&](int kt, int set) {  // set == kt & 1, a literal at both call sites
-    load_frags(set, 1, fa1, fb1);
-    mma(fa0, fb0);
-    __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above the barrier: they hide the reads
-    __syncthreads();
-    __builtin_amdgcn_sched_barrier(0);
-    if (kt + 1 < nk) load_frags(set ^ 1, 0, fa0, fb0);
-    if (kt + 2 < nk) {
-      lds_store(set, set);
-      if (kt + 4 < nk) global_fetch(kt + 4, set);
-    }
-    mma(fa1, fb1);
-  };
   int kt = 0;
-  for (; kt + 1 < nk; kt += 2) {  // no control flow around the MFMAs inside the loop
-    iteration(kt, 0);
-    iteration(kt + 1, 1);
+  if constexpr (GENERIC) {
+    // any K: run-time conditions inside the loop
+    auto iteration = [&](int kt, int stage) {
+      load_frags(stage, 1, fa1, fb1);
+      mma(fa0, fb0);
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+      if (kt + 1 < nk) load_frags(stage ^ 1, 0, fa0, fb0);
+      if (kt + 2 < nk) {
+        lds_store(stage);
+        if (kt + 3 < nk) global_fetch(kt + 3);
+      }
+      mma(fa1, fb1);
+    };
+    for (; kt + 1 < nk; kt += 2) {
+      iteration(kt, 0);
+      iteration(kt + 1, 1);
+    }
+    if (kt < nk) iteration(kt, 0);
+  } else {
+    // even nk >= 4: straight-line segments, no control flow around the MFMAs.  The
+    // sched_group_barrier sequences ask the scheduler to slot each LDS / global memory
+    // instruction between MFMAs, so their issue cycles hide under the matrix pipe.
+    // (masks: 0x008 MFMA, 0x100 LDS read, 0x200 LDS write, 0x020 global read)
+    constexpr int F_STORE = 1, F_FETCH = 2, F_NEXT = 4;
+    auto iteration = [&](int kt, auto stage_c, auto flags_c) {
+      constexpr int stage = decltype(stage_c)::value;
+      constexpr int F = decltype(flags_c)::value;
+      load_frags(stage, 1, fa1, fb1);
+      mma(fa0, fb0);
+#pragma unroll
+      for (int g = 0; g < TM + 4; ++g) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, TM / 2, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // the MFMAs stay above the barrier: they hide the reads
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr ((F & F_NEXT) != 0) load_frags(stage ^ 1, 0, fa0, fb0);
+      if constexpr ((F & F_STORE) != 0) lds_store(stage);
+      if constexpr ((F & F_FETCH) != 0) global_fetch(kt + 3);
+      mma(fa1, fb1);
+#pragma unroll
+      for (int g = 0; g < TM + 4; ++g) {
+        if constexpr ((F & F_NEXT) != 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, TM / 2, 0);
+        if constexpr ((F & F_STORE) != 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        if constexpr ((F & F_FETCH) != 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using All = std::integral_constant<int, F_STORE | F_FETCH | F_NEXT>;
+    for (; kt + 4 < nk; kt += 2) {
+      iteration(kt, S0{}, All{});
+      iteration(kt + 1, S1{}, All{});
+    }
+    iteration(kt, S0{}, All{});
+    iteration(kt + 1, S1{}, std::integral_constant<int, F_STORE | F_NEXT>{});
+    iteration(kt + 2, S0{}, std::integral_constant<int, F_NEXT>{});
+    iteration(kt + 3, S1{}, std::integral_constant<int, 0>{});
   }
-  if (kt < nk) iteration(kt, 0);  // odd number of k tiles
 
   // ---- epilogue: lane owns columns nc..nc+3 of rows (i, r) -------------------
   const int nc = n0 + wn * 128 + 4 * lr;
@@ -300,6 +361,8 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   SF_REQUIRE(xq && wq && out, "gemm_i8: null pointer");
   SF_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_i8: bad shape M=%lld N=%d K=%d", (long long)M, N, K);
   SF_REQUIRE(M < (1ll << 31) - 256, "gemm_i8: M=%lld too large", (long long)M);
+  SF_REQUIRE(M * K < (1ll << 31) && (int64_t)N * K < (1ll << 31),
+             "gemm_i8: operands of 2 GiB or more are not supported");
   SF_REQUIRE(K % GBK == 0, "gemm_i8: K=%d must be a multiple of %d", K, GBK);
   SF_REQUIRE(N % 8 == 0, "gemm_i8: N=%d must be a multiple of 8", N);
   SF_REQUIRE(ldo >= N, "gemm_i8: output row stride %lld < N=%d", (long long)ldo, N);
@@ -326,17 +389,23 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
     SF_REQUIRE(!dst_row || aligned16(dst_row), "gemm_i8: dst_row must be 16-byte aligned");
   }
   const char* force = getenv("SAMFAST_GEMM_TM");  // tuning aid: 2 or 4
-  const int tm = force ? atoi(force) : 2;
+  const bool generic_k = ((K / GBK) & 1) != 0 || K / GBK < 4;
+  const int tm = generic_k ? 2 : (force ? atoi(force) : 2);
   const int bm = 64 * tm;
   a.tiles_m = (int)((M + bm - 1) / bm);
   a.tiles_n = (N + GBN - 1) / GBN;
   const int64_t total = (int64_t)a.tiles_m * a.tiles_n;
   SF_REQUIRE(total < (1ll << 30), "gemm_i8: too many tiles");
   const unsigned int grid = (unsigned int)(((total + 7) / 8) * 8);
-#define SF_GEMM_LAUNCH(E)                                                                          \
-  do {                                                                                             \
-    if (tm == 4) hipLaunchKernelGGL((gemm_i8_kernel<E, 4>), dim3(grid), dim3(256), 0, stream, a);  \
-    else hipLaunchKernelGGL((gemm_i8_kernel<E, 2>), dim3(grid), dim3(256), 0, stream, a);          \
+  const bool generic = generic_k;
+#define SF_GEMM_LAUNCH(E)                                                                      \
+  do {                                                                                         \
+    if (generic)                                                                               \
+      hipLaunchKernelGGL((gemm_i8_kernel<E, 2, true>), dim3(grid), dim3(256), 0, stream, a);   \
+    else if (tm == 4)                                                                          \
+      hipLaunchKernelGGL((gemm_i8_kernel<E, 4, false>), dim3(grid), dim3(256), 0, stream, a);  \
+    else                                                                                       \
+      hipLaunchKernelGGL((gemm_i8_kernel<E, 2, false>), dim3(grid), dim3(256), 0, stream, a);  \
   } while (0)
   switch (epi) {
     case EPI_I32: SF_GEMM_LAUNCH(EPI_I32); break;
