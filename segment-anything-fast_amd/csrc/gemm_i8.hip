@@ -5,24 +5,31 @@
 //
 // Tiling: a 256-thread workgroup owns a (64*TM)x256 output tile; its four
 // wavefronts sit 2x2, each holding a (32*TM)x128 sub-tile as TMx4 MFMA tiles.
-// TM = 4 (256x256, 256 accumulator registers, one workgroup per CU) has the best
-// operand reuse; TM = 2 (128x256, 128 accumulators) lets two workgroups share a CU
-// so that the epilogue of one (a burst of HBM writes) runs under the MFMA loop of
-// the other.  K advances 64 bytes per iteration through two LDS stages with
-// global loads running two tiles ahead and the MFMA operand fragments of the next
-// k-step (also across the iteration boundary) read from LDS while the current
-// MFMAs execute; one barrier per iteration, placed between the two k-steps.  LDS rows
-// are 64 bytes with their four 16-byte chunks XOR-swizzled by the row index, so both
-// the tile writes and the operand reads are free of bank conflicts.
+// TM = 2 (128x256, 128 accumulators) is the default: two workgroups share a CU, so
+// the epilogue of one (a burst of HBM writes) runs under the MFMA loop of the other.
+// TM = 4 (256x256, one workgroup per CU) has better operand reuse but no such overlap
+// and measures slower at the encoder's shapes.
 //
-// W rows are stored in LDS in a permuted order (row n of a wave's 128 columns
-// goes to slot (n%4)*32 + n/4) so that MFMA tile j, lane-column c holds output
-// column 4c+j: after the K loop every lane owns 4 adjacent columns of each of its
-// rows and writes them with one 8-byte (bf16) or 16-byte (int32) store.
+// K loop (main kernel, K >= 256): tiles of 64 bytes of K travel global memory -> LDS
+// directly (global_load_lds_dwordx4: no staging registers, no LDS write instructions)
+// through three (TM = 2) or four (TM = 4) LDS stages; in-order completion of vector
+// memory loads lets "tile kt+1 has landed" be a vmcnt threshold that leaves later tiles
+// in flight across the one barrier per iteration.  The MFMA operand fragments of the
+// next 32-byte k-step - also across the iteration boundary - are read from LDS while
+// the current MFMAs execute, and sched_group_barrier sequences slot every LDS / global
+// instruction between MFMAs.  LDS rows are 64 bytes with their four 16-byte chunks
+// XOR-swizzled by the row index: tile writes and operand reads are bank-conflict free
+// (SQ_LDS_BANK_CONFLICT = 0).  A small register-staged variant of the same loop handles
+// K < 256.
 //
-// Workgroup ids are first made contiguous per XCD, then walked in groups of 8
-// row-panels x all column tiles so that the tiles resident on one XCD share
-// their X panels and the W matrix in that XCD's L2.
+// W rows are stored in LDS in a permuted order (slot s of a wave's 128 columns holds
+// row (s%32)*4 + s/32) so that MFMA tile j, lane-column c holds output column 4c+j:
+// after the K loop every lane owns 4 adjacent columns of each of its rows and writes
+// them with one 8-byte (bf16) or 16-byte (int32) store.
+//
+// Workgroup ids are first made contiguous per XCD, then walked in groups of 2048 output
+// rows x all column tiles so that the tiles resident on one XCD share their X panels
+// and the W matrix in that XCD's L2.
 #include "samfast_internal.hpp"
 #include <stdlib.h>
 #include <type_traits>
@@ -69,193 +76,11 @@ SF_DEVICE float gelu_erf(float x) {
   return x * phi;
 }
 
-// 16-byte chunk c of LDS row r lives at chunk position c ^ lds_swizzle(r).  With it the
-// operand reads (one chunk of 8 / 16 consecutive rows per LDS cycle) and the tile writes
-// (4 chunks of 2 / 4 consecutive rows per cycle) both touch every bank once, whether the
-// LDS cycles through 128 or 256 bytes.
-SF_DEVICE int lds_swizzle(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
-
-template <int EPI, int TM, bool GENERIC>
-__global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArgs a) {
-  constexpr int GBM = 64 * TM;
-  constexpr int GSTAGE = (GBM + GBN) * GLD;
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * GSTAGE];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int lr = lane & 31, lh = lane >> 5;
-
-  const unsigned int total = (unsigned int)a.tiles_m * (unsigned int)a.tiles_n;
-  const unsigned int pid = xcd_contiguous_id(blockIdx.x, total);
-  if (pid >= total) return;  // uniform over the workgroup
-  constexpr int GGROUP_M = 32 / TM;  // 2048 output rows per group
-  const unsigned int per_group = GGROUP_M * a.tiles_n;
-  const unsigned int first_m = (pid / per_group) * GGROUP_M;
-  const unsigned int gsz = min((unsigned int)a.tiles_m - first_m, (unsigned int)GGROUP_M);
-  const unsigned int in_group = pid % per_group;
-  const int m0 = (int)(first_m + in_group % gsz) * GBM;
-  const int n0 = (int)(in_group / gsz) * GBN;
-
-  // ---- global -> LDS staging: 16-byte chunks, TM per thread for X and 4 for W ----
-  // (32-bit lane offsets from the uniform matrix bases; M*K and N*K fit in 31 bits)
-  int ox[TM], ow[4];
-  int lx[TM], lw[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int c = tid + 256 * i;
-    const int row = c >> 2, kc = c & 3;
-    if (i < TM) {
-      const int gm = min(m0 + row, a.M - 1);
-      ox[i] = gm * a.K + kc * 16;
-      lx[i] = row * GLD + ((kc ^ lds_swizzle(row)) * 16);
-    }
-    // W: consecutive chunk groups go to consecutive LDS slots (no write bank conflicts);
-    // slot s of a 128-column half holds W row (s % 32) * 4 + s / 32 of that half
-    const int slot = row & 127;
-    const int wrow = (row & 128) + (slot & 31) * 4 + (slot >> 5);
-    const int gn = min(n0 + wrow, a.N - 1);
-    ow[i] = gn * a.K + kc * 16;
-    lw[i] = GBM * GLD + row * GLD + ((kc ^ lds_swizzle(row)) * 16);
-  }
-
-  i32x16 acc[TM][4];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
-  // ---- software pipeline -------------------------------------------------------
-  // Two LDS stages, the barrier in the MIDDLE of an iteration.  Iteration kt:
-  //   A. read the fragments of k-step 1 of tile kt (stage kt&1) while the MFMAs of
-  //      k-step 0 run;
-  //   B. barrier: every wave now holds all of tile kt in registers, so stage kt&1 is
-  //      free, and tile kt+1 (written in the previous iteration) is visible;
-  //   C. read the fragments of k-step 0 of tile kt+1, write tile kt+2 (fetched from
-  //      global memory into registers one iteration ago) into the freed stage, issue
-  //      the global loads of tile kt+3 - all while the MFMAs of k-step 1 run.
-  i32x4 stg_x[TM], stg_w[4];
-  auto global_fetch = [&](int kt) {
-    const int8_t* xb = a.x + kt * GBK;  // uniform
-    const int8_t* wb = a.w + kt * GBK;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (i < TM) stg_x[i] = *reinterpret_cast<const i32x4*>(xb + ox[i]);
-      stg_w[i] = *reinterpret_cast<const i32x4*>(wb + ow[i]);
-    }
-  };
-  auto lds_store = [&](int stage) {
-    unsigned char* dst = lds + stage * GSTAGE;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (i < TM) *reinterpret_cast<i32x4*>(dst + lx[i]) = stg_x[i];
-      *reinterpret_cast<i32x4*>(dst + lw[i]) = stg_w[i];
-    }
-  };
-  // fragment of k-step s: chunk 2s + lh of row (tile row base + lr); the swizzle only
-  // depends on lr because every tile row base is a multiple of 32
-  const int frag_chunk = (lh ^ lds_swizzle(lr)) * 16;
-  const int a_off = (wm * 32 * TM + lr) * GLD + frag_chunk;
-  const int b_off = GBM * GLD + (wn * 128 + lr) * GLD + frag_chunk;
-  auto load_frags = [&](int stage, int step, i32x4 (&av)[TM], i32x4 (&bv)[4]) {
-    const unsigned char* src = lds + stage * GSTAGE;
-    const int flip = step * 32;  // (2*step + lh) ^ swz == ((lh ^ swz) ^ 2*step) as a chunk index
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (i < TM) av[i] = *reinterpret_cast<const i32x4*>(src + ((a_off + i * 32 * GLD) ^ flip));
-      bv[i] = *reinterpret_cast<const i32x4*>(src + ((b_off + i * 32 * GLD) ^ flip));
-    }
-  };
-  auto mma = [&](const i32x4 (&av)[TM], const i32x4 (&bv)[4]) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], acc[i][j], 0, 0, 0);
-  };
-
-  const int nk = a.K / GBK;
-  global_fetch(0);
-  lds_store(0);
-  if (nk > 1) {
-    global_fetch(1);
-    lds_store(1);
-  }
-  if (nk > 2) global_fetch(2);
-  __syncthreads();
-
-  i32x4 fa0[TM], fb0[4], fa1[TM], fb1[4];
-  load_frags(0, 0, fa0, fb0);
-  int kt = 0;
-  if constexpr (GENERIC) {
-    // any K: run-time conditions inside the loop
-    auto iteration = [&](int kt, int stage) {
-      load_frags(stage, 1, fa1, fb1);
-      mma(fa0, fb0);
-      __builtin_amdgcn_sched_barrier(0);
-      __syncthreads();
-      __builtin_amdgcn_sched_barrier(0);
-      if (kt + 1 < nk) load_frags(stage ^ 1, 0, fa0, fb0);
-      if (kt + 2 < nk) {
-        lds_store(stage);
-        if (kt + 3 < nk) global_fetch(kt + 3);
-      }
-      mma(fa1, fb1);
-    };
-    for (; kt + 1 < nk; kt += 2) {
-      iteration(kt, 0);
-      iteration(kt + 1, 1);
-    }
-    if (kt < nk) iteration(kt, 0);
-  } else {
-    // even nk >= 4: straight-line segments, no control flow around the MFMAs.  The
-    // sched_group_barrier sequences ask the scheduler to slot each LDS / global memory
-    // instruction between MFMAs, so their issue cycles hide under the matrix pipe.
-    // (masks: 0x008 MFMA, 0x100 LDS read, 0x200 LDS write, 0x020 global read)
-    constexpr int F_STORE = 1, F_FETCH = 2, F_NEXT = 4;
-    auto iteration = [&](int kt, auto stage_c, auto flags_c) {
-      constexpr int stage = decltype(stage_c)::value;
-      constexpr int F = decltype(flags_c)::value;
-      load_frags(stage, 1, fa1, fb1);
-      mma(fa0, fb0);
-#pragma unroll
-      for (int g = 0; g < TM + 4; ++g) {
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, TM / 2, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);  // the MFMAs stay above the barrier: they hide the reads
-      __syncthreads();
-      __builtin_amdgcn_sched_barrier(0);
-      if constexpr ((F & F_NEXT) != 0) load_frags(stage ^ 1, 0, fa0, fb0);
-      if constexpr ((F & F_STORE) != 0) lds_store(stage);
-      if constexpr ((F & F_FETCH) != 0) global_fetch(kt + 3);
-      mma(fa1, fb1);
-#pragma unroll
-      for (int g = 0; g < TM + 4; ++g) {
-        if constexpr ((F & F_NEXT) != 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, TM / 2, 0);
-        if constexpr ((F & F_STORE) != 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-        if constexpr ((F & F_FETCH) != 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    using S0 = std::integral_constant<int, 0>;
-    using S1 = std::integral_constant<int, 1>;
-    using All = std::integral_constant<int, F_STORE | F_FETCH | F_NEXT>;
-    for (; kt + 4 < nk; kt += 2) {
-      iteration(kt, S0{}, All{});
-      iteration(kt + 1, S1{}, All{});
-    }
-    iteration(kt, S0{}, All{});
-    iteration(kt + 1, S1{}, std::integral_constant<int, F_STORE | F_NEXT>{});
-    iteration(kt + 2, S0{}, std::integral_constant<int, F_NEXT>{});
-    iteration(kt + 3, S1{}, std::integral_constant<int, 0>{});
-  }
-
-  // ---- epilogue: lane owns columns nc..nc+3 of rows (i, r) -------------------
+// Epilogue shared by the kernels: the lane owns 4 adjacent output columns of each of
+// its 16*TM rows (MFMA tile i, register r -> row i*32 + 8*(r/4) + 4*lh + r%4).
+template <int EPI, int TM>
+SF_DEVICE void gemm_epilogue(const GemmArgs& a, i32x16 (&acc)[TM][4], int m0, int n0, int wm,
+                             int wn, int lr, int lh) {
   const int nc = n0 + wn * 128 + 4 * lr;
   if (nc >= a.N) return;  // N % 8 == 0, so a lane's 4 columns are in or out together
   const int mrow0 = m0 + wm * 32 * TM + 4 * lh;  // + i*32 + 8*(r>>2) + (r&3)
@@ -354,6 +179,254 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
   }
 }
 
+// 16-byte chunk c of LDS row r lives at chunk position c ^ lds_swizzle(r).  With it the
+// operand reads (one chunk of 8 / 16 consecutive rows per LDS cycle) and the tile writes
+// (4 chunks of 2 / 4 consecutive rows per cycle) both touch every bank once, whether the
+// LDS cycles through 128 or 256 bytes.
+SF_DEVICE int lds_swizzle(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
+
+template <int EPI, int TM, bool GENERIC>
+__global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArgs a) {
+  constexpr int GBM = 64 * TM;
+  constexpr int GSTAGE = (GBM + GBN) * GLD;
+  constexpr int NST = GENERIC ? 2 : (TM == 4 ? 4 : 3);  // LDS stages
+  __shared__ __attribute__((aligned(16))) unsigned char lds[NST * GSTAGE];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lr = lane & 31, lh = lane >> 5;
+
+  const unsigned int total = (unsigned int)a.tiles_m * (unsigned int)a.tiles_n;
+  const unsigned int pid = xcd_contiguous_id(blockIdx.x, total);
+  if (pid >= total) return;  // uniform over the workgroup
+  constexpr int GGROUP_M = 32 / TM;  // 2048 output rows per group
+  const unsigned int per_group = GGROUP_M * a.tiles_n;
+  const unsigned int first_m = (pid / per_group) * GGROUP_M;
+  const unsigned int gsz = min((unsigned int)a.tiles_m - first_m, (unsigned int)GGROUP_M);
+  const unsigned int in_group = pid % per_group;
+  const int m0 = (int)(first_m + in_group % gsz) * GBM;
+  const int n0 = (int)(in_group / gsz) * GBN;
+
+  // ---- global -> LDS staging: 16-byte chunks, TM per thread for X and 4 for W ----
+  // (32-bit lane offsets from the uniform matrix bases; M*K and N*K fit in 31 bits)
+  int ox[TM], ow[4];
+  int lx[TM], lw[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = tid + 256 * i;
+    const int row = c >> 2, kc = c & 3;
+    if (i < TM) {
+      const int gm = min(m0 + row, a.M - 1);
+      ox[i] = gm * a.K + kc * 16;
+      lx[i] = row * GLD + ((kc ^ lds_swizzle(row)) * 16);
+    }
+    // W: consecutive chunk groups go to consecutive LDS slots (no write bank conflicts);
+    // slot s of a 128-column half holds W row (s % 32) * 4 + s / 32 of that half
+    const int slot = row & 127;
+    const int wrow = (row & 128) + (slot & 31) * 4 + (slot >> 5);
+    const int gn = min(n0 + wrow, a.N - 1);
+    ow[i] = gn * a.K + kc * 16;
+    lw[i] = GBM * GLD + row * GLD + ((kc ^ lds_swizzle(row)) * 16);
+  }
+
+  i32x16 acc[TM][4];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  // ---- software pipeline -------------------------------------------------------
+  // Two LDS stages, the barrier in the MIDDLE of an iteration.  Iteration kt:
+  //   A. read the fragments of k-step 1 of tile kt (stage kt&1) while the MFMAs of
+  //      k-step 0 run;
+  //   B. barrier: every wave now holds all of tile kt in registers, so stage kt&1 is
+  //      free, and tile kt+1 (written in the previous iteration) is visible;
+  //   C. read the fragments of k-step 0 of tile kt+1, write tile kt+2 (fetched from
+  //      global memory into registers one iteration ago) into the freed stage, issue
+  //      the global loads of tile kt+3 - all while the MFMAs of k-step 1 run.
+  i32x4 stg_x[TM], stg_w[4];
+  auto global_fetch = [&](int kt) {
+    const int8_t* xb = a.x + kt * GBK;  // uniform
+    const int8_t* wb = a.w + kt * GBK;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (i < TM) stg_x[i] = *reinterpret_cast<const i32x4*>(xb + ox[i]);
+      stg_w[i] = *reinterpret_cast<const i32x4*>(wb + ow[i]);
+    }
+  };
+  auto lds_store = [&](int stage) {
+    unsigned char* dst = lds + stage * GSTAGE;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (i < TM) *reinterpret_cast<i32x4*>(dst + lx[i]) = stg_x[i];
+      *reinterpret_cast<i32x4*>(dst + lw[i]) = stg_w[i];
+    }
+  };
+  // fragment of k-step s: chunk 2s + lh of row (tile row base + lr); the swizzle only
+  // depends on lr because every tile row base is a multiple of 32
+  const int frag_chunk = (lh ^ lds_swizzle(lr)) * 16;
+  const int a_off = (wm * 32 * TM + lr) * GLD + frag_chunk;
+  const int b_off = GBM * GLD + (wn * 128 + lr) * GLD + frag_chunk;
+  auto load_frags = [&](int stage, int step, i32x4 (&av)[TM], i32x4 (&bv)[4]) {
+    const unsigned char* src = lds + stage * GSTAGE;
+    const int flip = step * 32;  // (2*step + lh) ^ swz == ((lh ^ swz) ^ 2*step) as a chunk index
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (i < TM) av[i] = *reinterpret_cast<const i32x4*>(src + ((a_off + i * 32 * GLD) ^ flip));
+      bv[i] = *reinterpret_cast<const i32x4*>(src + ((b_off + i * 32 * GLD) ^ flip));
+    }
+  };
+  auto mma = [&](const i32x4 (&av)[TM], const i32x4 (&bv)[4]) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], acc[i][j], 0, 0, 0);
+  };
+
+  const int nk = a.K / GBK;
+  i32x4 fa0[TM], fb0[4], fa1[TM], fb1[4];
+  int kt = 0;
+  if constexpr (GENERIC) {
+    global_fetch(0);
+    lds_store(0);
+    if (nk > 1) {
+      global_fetch(1);
+      lds_store(1);
+    }
+    if (nk > 2) global_fetch(2);
+    __syncthreads();
+    load_frags(0, 0, fa0, fb0);
+    // any K: run-time conditions inside the loop
+    auto iteration = [&](int kt, int stage) {
+      load_frags(stage, 1, fa1, fb1);
+      mma(fa0, fb0);
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+      if (kt + 1 < nk) load_frags(stage ^ 1, 0, fa0, fb0);
+      if (kt + 2 < nk) {
+        lds_store(stage);
+        if (kt + 3 < nk) global_fetch(kt + 3);
+      }
+      mma(fa1, fb1);
+    };
+    for (; kt + 1 < nk; kt += 2) {
+      iteration(kt, 0);
+      iteration(kt + 1, 1);
+    }
+    if (kt < nk) iteration(kt, 0);
+  } else {
+    // nk >= 4.  Tiles travel global memory -> LDS directly (global_load_lds_dwordx4, no
+    // staging registers, no LDS write instructions) through THREE stages, so a tile has
+    // two full iterations to arrive.  One wave instruction fills 1 KB = 16 LDS rows; lane l
+    // lands at chunk position l&3 of row l>>2 of that block, so the XOR swizzle is applied
+    // to the GLOBAL address (the lane fetches the chunk that belongs at its position).
+    // In-order completion lets "tile kt+1 has landed" be expressed as vmcnt <= (loads per
+    // tile), leaving tile kt+2 in flight across the barrier.
+    constexpr int NLD = (GBM + GBN) / 64;  // wave instructions per tile and wave: 6 / 8
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    int dma_off[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const int rho = 16 * (wave_u + 4 * i) + (lane >> 2);  // LDS row of this lane's chunk
+      const int chunk = (lane & 3) ^ lds_swizzle(rho);
+      if (i < GBM / 64) {  // X rows
+        dma_off[i] = min(m0 + rho, a.M - 1) * a.K + chunk * 16;
+      } else {             // W slots (slot s of a 128-column half holds W row (s%32)*4 + s/32)
+        const int sl = rho - GBM;
+        const int wrow = (sl & 128) + (sl & 31) * 4 + ((sl & 127) >> 5);
+        dma_off[i] = min(n0 + wrow, a.N - 1) * a.K + chunk * 16;
+      }
+    }
+    typedef __attribute__((address_space(1))) const void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    auto dma_issue = [&](int kt, int stage_off) {
+      const int8_t* xb = a.x + kt * GBK;
+      const int8_t* wb = a.w + kt * GBK;
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int8_t* src = (i < GBM / 64 ? xb : wb) + dma_off[i];
+        unsigned char* dst = lds + stage_off + (wave_u + 4 * i) * 1024;
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
+      }
+    };
+    auto frags_at = [&](int stage_off, int step, i32x4 (&av)[TM], i32x4 (&bv)[4]) {
+      const unsigned char* src = lds + stage_off;
+      const int flip = step * 32;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (i < TM) av[i] = *reinterpret_cast<const i32x4*>(src + ((a_off + i * 32 * GLD) ^ flip));
+        bv[i] = *reinterpret_cast<const i32x4*>(src + ((b_off + i * 32 * GLD) ^ flip));
+      }
+    };
+    // s_waitcnt immediate: vmcnt in bits 3:0 and 15:14 ("at most n loads still in flight"),
+    // expcnt 6:4 = 7 (no wait), lgkmcnt 11:8 = 0 (all of this wave's LDS reads done)
+    auto wait_imm = [](int n) constexpr { return 0x0070 | (n & 15) | ((n >> 4) << 14); };
+    static_assert((NST - 1) * NLD <= 63, "vmcnt immediate");
+
+    int st[NST];  // st[j] = LDS offset of the stage holding tile kt + j (uniform, rotated)
+#pragma unroll
+    for (int j = 0; j < NST; ++j) {
+      st[j] = j * GSTAGE;
+      dma_issue(j, st[j]);  // nk >= NST is guaranteed by the host
+    }
+    __builtin_amdgcn_s_waitcnt(wait_imm((NST - 1) * NLD));
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    frags_at(st[0], 0, fa0, fb0);
+
+    // ISSUE: fetch tile kt+NST into the stage freed at the barrier; NEXT: a tile kt+1
+    // exists; KEEP: tiles that may stay in flight across the barrier (after tile kt+1).
+    // (sched_group_barrier masks: 0x008 MFMA, 0x100 LDS read, 0x020 global read)
+    auto iteration = [&](int kt, auto issue_c, auto next_c, auto keep_c) {
+      constexpr bool ISSUE = decltype(issue_c)::value != 0;
+      constexpr bool NEXT = decltype(next_c)::value != 0;
+      constexpr int KEEP = decltype(keep_c)::value;
+      frags_at(st[0], 1, fa1, fb1);
+      mma(fa0, fb0);
+#pragma unroll
+      for (int g = 0; g < TM + 4; ++g) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, TM / 2, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // own LDS reads of this stage done; own share of tile kt+1 landed; then all waves meet
+      __builtin_amdgcn_s_waitcnt(wait_imm(KEEP * NLD));
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (ISSUE) dma_issue(kt + NST, st[0]);
+      if constexpr (NEXT) frags_at(st[1], 0, fa0, fb0);
+      mma(fa1, fb1);
+#pragma unroll
+      for (int g = 0; g < TM + 4; ++g) {
+        if constexpr (NEXT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, TM / 2, 0);
+        if constexpr (ISSUE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const int t = st[0];
+#pragma unroll
+      for (int j = 0; j + 1 < NST; ++j) st[j] = st[j + 1];
+      st[NST - 1] = t;
+    };
+    using Yes = std::integral_constant<int, 1>;
+    using No = std::integral_constant<int, 0>;
+    for (; kt + NST < nk; ++kt) iteration(kt, Yes{}, Yes{}, std::integral_constant<int, NST - 2>{});
+    // the last NST iterations fetch nothing; fewer and fewer tiles remain in flight
+    if constexpr (NST == 4) iteration(kt++, No{}, Yes{}, std::integral_constant<int, 2>{});
+    iteration(kt++, No{}, Yes{}, std::integral_constant<int, 1>{});
+    iteration(kt++, No{}, Yes{}, No{});
+    iteration(kt++, No{}, No{}, No{});
+  }
+
+  gemm_epilogue<EPI, TM>(a, acc, m0, n0, wm, wn, lr, lh);
+}
+
 static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t* wq,
                        const float* sw, const float* bias, void* out, int64_t ldo, int64_t M,
                        int N, int K, hipStream_t stream, const void* residual = nullptr,
@@ -389,8 +462,8 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
     SF_REQUIRE(!dst_row || aligned16(dst_row), "gemm_i8: dst_row must be 16-byte aligned");
   }
   const char* force = getenv("SAMFAST_GEMM_TM");  // tuning aid: 2 or 4
-  const bool generic_k = ((K / GBK) & 1) != 0 || K / GBK < 4;
-  const int tm = generic_k ? 2 : (force ? atoi(force) : 2);
+  const bool generic_k = K / GBK < 4;  // fewer k tiles than LDS stages
+  const int tm = generic_k ? 2 : (force && atoi(force) == 4 ? 4 : 2);
   const int bm = 64 * tm;
   a.tiles_m = (int)((M + bm - 1) / bm);
   a.tiles_n = (N + GBN - 1) / GBN;
