@@ -27,7 +27,7 @@
 // after the K loop every lane owns 4 adjacent columns of each of its rows and writes
 // them with one 8-byte (bf16) or 16-byte (int32) store.
 //
-// Workgroup ids are first made contiguous per XCD, then walked in groups of 2048 output
+// Workgroup ids are first made contiguous per XCD, then walked in groups of 1024 output
 // rows x all column tiles so that the tiles resident on one XCD share their X panels
 // and the W matrix in that XCD's L2.
 #include "samfast_internal.hpp"
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
   const unsigned int total = (unsigned int)a.tiles_m * (unsigned int)a.tiles_n;
   const unsigned int pid = xcd_contiguous_id(blockIdx.x, total);
   if (pid >= total) return;  // uniform over the workgroup
-  constexpr int GGROUP_M = 32 / TM;  // 2048 output rows per group
+  constexpr int GGROUP_M = 16 / TM;  // 1024 output rows per group: their X panels (1.3 MB at K=1280) stay in L2
   const unsigned int per_group = GGROUP_M * a.tiles_n;
   const unsigned int first_m = (pid / per_group) * GGROUP_M;
   const unsigned int gsz = min((unsigned int)a.tiles_m - first_m, (unsigned int)GGROUP_M);
