@@ -60,22 +60,6 @@ struct GemmArgs {
   const int32_t* dst_row;          // EPI_RESIDUAL: output row per GEMM row, -1 = drop; may be null
 };
 
-// x * Phi(x) with Phi from the Abramowitz-Stegun 7.1.26 erfc polynomial (|error| <
-// 1.5e-7), evaluated as erfc on the negative side so the tail keeps its relative accuracy.
-SF_DEVICE float gelu_erf(float x) {
-#pragma clang fp contract(fast)  // an approximation anyway: let the polynomial use FMAs
-  const float z = fabsf(x) * 0.70710678118654752f;
-  const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
-  float poly = 1.061405429f;
-  poly = poly * t + -1.453152027f;
-  poly = poly * t + 1.421413741f;
-  poly = poly * t + -0.284496736f;
-  poly = poly * t + 0.254829592f;
-  const float half_erfc = 0.5f * poly * t * __builtin_amdgcn_exp2f(-1.4426950408889634f * z * z);
-  const float phi = x >= 0.f ? 1.0f - half_erfc : half_erfc;
-  return x * phi;
-}
-
 // Epilogue shared by the kernels: the lane owns 4 adjacent output columns of each of
 // its 16*TM rows (MFMA tile i, register r -> row i*32 + 8*(r/4) + 4*lh + r%4).
 template <int EPI, int TM>

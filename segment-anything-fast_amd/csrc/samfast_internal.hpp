@@ -62,6 +62,25 @@ SF_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 // value held by lane (lane ^ 32) of the same wavefront
 SF_DEVICE float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
+// GELU(x) = x * Phi(x) with 1 - Phi(|x|) = 0.5 * erfc(|x| / sqrt 2) from the
+// Abramowitz-Stegun 7.1.26 polynomial (|error| < 1.5e-7), written so that the negative
+// side keeps its relative accuracy:  gelu(x) = max(x, 0) - |x| * h,
+//   h = 0.5 * poly(t) * exp(-x^2 / 2),  t = 1 / (1 + p |x| / sqrt 2).
+SF_DEVICE float gelu_erf(float x) {
+#pragma clang fp contract(fast)  // an approximation anyway: let the polynomial use FMAs
+  const float ax = fabsf(x);
+  const float t = __builtin_amdgcn_rcpf(fmaf(ax, 0.3275911f * 0.70710678118654752f, 1.0f));
+  const float w = ax * 0.84932180028801904f;  // sqrt(log2(e) / 2): exp(-x^2/2) = exp2(-w^2)
+  const float e = __builtin_amdgcn_exp2f(-(w * w));
+  float poly = 0.5f * 1.061405429f;            // the 0.5 of h is folded into the coefficients
+  poly = fmaf(poly, t, 0.5f * -1.453152027f);
+  poly = fmaf(poly, t, 0.5f * 1.421413741f);
+  poly = fmaf(poly, t, 0.5f * -0.284496736f);
+  poly = fmaf(poly, t, 0.5f * 0.254829592f);
+  const float h = poly * t * e;
+  return fmaf(-ax, h, fmaxf(x, 0.f));
+}
+
 // Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its
 // own L2.  Map the hardware id to a logical id so that every XCD walks one
 // contiguous range of logical ids (neighbours then share an L2).
