@@ -165,6 +165,44 @@ int samfast_gemm_i8_fused(
     int64_t M, int N, int K, int dtype, int epilogue,
     const void* residual, int64_t ld_res, const int32_t* dst_row, void* stream);
 
+/*
+ * 2:4-sparse weights for the sparse int8 matrix cores (v_smfmac_i32_32x32x64_i8).
+ *
+ * samfast_prune24_pack_i8: from a dense int8 weight wq (N, K) keep, in every aligned group
+ * of 4 consecutive k, the 2 entries of largest magnitude (ties: lowest k) and write them in
+ * the packed form the GEMM below reads.  A matrix that already is 2:4 (at most 2 non-zeros
+ * per group, e.g. quantised after magnitude pruning of the float weight) is packed without
+ * loss.  K % 64 == 0.  Packed layout, K-block major (kb = k / 64):
+ *   wc   (K/64, N, 32) int8:  byte 16*h + 2*g + e  (h in 0..1, g in 0..7, e in 0..1) holds
+ *        wq[n, 64*kb + 32*(g/4) + 16*h + 4*(g%4) + p_e], p_0 < p_1 the kept positions;
+ *   widx (K/64, N, 2) int32:  word h, bits 4g+1:4g = p_0, bits 4g+3:4g+2 = p_1.
+ * Stands for the prune + compress steps of apply_sparse (sparse.py:6-32: WeightNormSparsifier
+ * with sparse_block_shape (1,4), zeros_per_block 2, then to_sparse_semi_structured), applied
+ * to int8 weights.
+ */
+int samfast_prune24_pack_i8(
+    const int8_t* wq, int8_t* wc, int32_t* widx, int N, int K, void* stream);
+
+/*
+ * acc[m, n] = sum_k xq[m, k] * w[n, k] (int32, exact) with w given in the packed 2:4 form;
+ * equals samfast_gemm_i8_i32 on the pruned dense matrix.  K % 128 == 0, K >= 256, N % 8 == 0.
+ */
+int samfast_gemm_i8_sparse24_i32(
+    const int8_t* xq, const int8_t* wc, const int32_t* widx, int32_t* acc,
+    int64_t M, int N, int K, void* stream);
+
+/*
+ * samfast_gemm_i8_fused (epilogues NONE / GELU / RESIDUAL, no row scatter) with the weight
+ * in the packed 2:4 form: the semi-structured Linear the reference builds at sparse.py:28-32,
+ * here for the int8 MLP linears lin1 (GELU) and lin2 (residual) (modeling/common.py:26).
+ * y and residual rows must be 16-byte aligned (ldy, ld_res multiples of 8).
+ */
+int samfast_gemm_i8_sparse24_fused(
+    const int8_t* xq, const float* sx, const int8_t* wc, const int32_t* widx,
+    const float* sw, const float* bias, void* y, int64_t ldy,
+    int64_t M, int N, int K, int dtype, int epilogue,
+    const void* residual, int64_t ld_res, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

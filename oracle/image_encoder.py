@@ -70,8 +70,9 @@ def layer_norm_2d(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps
 
 def block_forward(sd: Dict[str, torch.Tensor], prefix: str, x: torch.Tensor,
                   cfg: EncoderConfig, window_size: int, linear=F.linear,
-                  use_sdpa: bool = False) -> torch.Tensor:
+                  use_sdpa: bool = False, mlp_linear=None) -> torch.Tensor:
     """One transformer block on (B, H, W, C); image_encoder.py:167-183."""
+    mlp_linear = mlp_linear or linear
     C = cfg.embed_dim
     p = lambda name: sd[prefix + name]
     shortcut = x
@@ -88,19 +89,20 @@ def block_forward(sd: Dict[str, torch.Tensor], prefix: str, x: torch.Tensor,
         y = ra.window_unpartition(y, window_size, pad_hw, (H, W))
     x = shortcut + y
     z = F.layer_norm(x, (C,), p("norm2.weight"), p("norm2.bias"), cfg.ln_eps)
-    z = linear(z, p("mlp.lin1.weight"), p("mlp.lin1.bias"))
+    z = mlp_linear(z, p("mlp.lin1.weight"), p("mlp.lin1.bias"))
     z = F.gelu(z)  # exact erf GELU, the nn.GELU default (common.py:17)
-    z = linear(z, p("mlp.lin2.weight"), p("mlp.lin2.bias"))
+    z = mlp_linear(z, p("mlp.lin2.weight"), p("mlp.lin2.bias"))
     return x + z
 
 
 def encoder_forward(sd: Dict[str, torch.Tensor], images: torch.Tensor, cfg: EncoderConfig,
-                    linear=F.linear, use_sdpa: bool = False) -> torch.Tensor:
+                    linear=F.linear, use_sdpa: bool = False, mlp_linear=None) -> torch.Tensor:
     """(B, 3, 1024, 1024) normalised images -> (B, 256, 64, 64) embeddings.
 
     `linear(x, w, b)` is used for the four Linears of every block (qkv, proj,
     lin1, lin2) - pass oracle.quant_linear.dynamic_int8_linear for the
-    quantised path.  Patch embedding and neck are convolutions and stay float.
+    quantised path.  `mlp_linear`, if given, replaces it for lin1 / lin2 only (the
+    2:4-sparse MLP configuration).  Patch embedding and neck are convolutions and stay float.
     use_sdpa=True routes attention through F.scaled_dot_product_attention with a
     materialised bias, which is what the reference executes on a CPU
     (flash_4.py:368-370); the default writes the softmax out.
@@ -112,7 +114,7 @@ def encoder_forward(sd: Dict[str, torch.Tensor], images: torch.Tensor, cfg: Enco
         x = x + sd["pos_embed"]
     for i in range(cfg.depth):
         ws = 0 if i in cfg.global_attn_indexes else cfg.window_size
-        x = block_forward(sd, f"blocks.{i}.", x, cfg, ws, linear, use_sdpa)
+        x = block_forward(sd, f"blocks.{i}.", x, cfg, ws, linear, use_sdpa, mlp_linear)
     x = x.permute(0, 3, 1, 2)
     x = F.conv2d(x, sd["neck.0.weight"])
     x = layer_norm_2d(x, sd["neck.1.weight"], sd["neck.1.bias"])

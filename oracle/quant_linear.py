@@ -122,3 +122,62 @@ def prune_2_of_4(weight: torch.Tensor) -> torch.Tensor:
     np.put_along_axis(keep, order[..., :2], True, axis=-1)
     out = (w.reshape(N, K // 4, 4) * keep).reshape(N, K)
     return torch.from_numpy(out).to(weight.dtype if isinstance(weight, torch.Tensor) else torch.float32)
+
+
+def _group_dense_offset(g: int, h: int) -> int:
+    """First dense k (inside a 64-wide block) of group g of lane half h, as the gfx950
+    sparse matrix instruction v_smfmac_i32_32x32x64_i8 pairs stored A bytes with B."""
+    return 32 * (g // 4) + 16 * h + 4 * (g % 4)
+
+
+def pack_2_of_4(wq: np.ndarray):
+    """Packed form of an int8 (N, K) matrix for the sparse int8 GEMM (layout documented at
+    samfast_prune24_pack_i8 in include/samfast.h): per aligned group of 4 along K the two
+    largest magnitudes (ties: lowest position) are kept.  The compress step of
+    segment_anything_fast/sparse.py:32 (to_sparse_semi_structured), restated for int8 and
+    the gfx950 operand order.  Pure-Python loops: small matrices only.
+
+    Returns (wc int8 (K/64, N, 32), widx int32 (K/64, N, 2)).
+    """
+    assert wq.dtype == np.int8 and wq.ndim == 2 and wq.shape[1] % 64 == 0
+    N, K = wq.shape
+    wc = np.zeros((K // 64, N, 32), dtype=np.int8)
+    widx = np.zeros((K // 64, N, 2), dtype=np.uint32)
+    for kb in range(K // 64):
+        for n in range(N):
+            for h in range(2):
+                word = 0
+                for g in range(8):
+                    base = 64 * kb + _group_dense_offset(g, h)
+                    grp = wq[n, base:base + 4].astype(np.int32)
+                    order = sorted(range(4), key=lambda p: (-abs(int(grp[p])), p))
+                    p0, p1 = sorted(order[:2])
+                    wc[kb, n, 16 * h + 2 * g] = grp[p0]
+                    wc[kb, n, 16 * h + 2 * g + 1] = grp[p1]
+                    word |= (p0 | (p1 << 2)) << (4 * g)
+                widx[kb, n, h] = word
+    return wc, widx.view(np.int32)
+
+
+def unpack_2_of_4(wc: np.ndarray, widx: np.ndarray) -> np.ndarray:
+    """Inverse of pack_2_of_4: the dense int8 (N, K) matrix a packed weight stands for."""
+    KB, N, _ = wc.shape
+    out = np.zeros((N, KB * 64), dtype=np.int8)
+    words = widx.view(np.uint32)
+    for kb in range(KB):
+        for n in range(N):
+            for h in range(2):
+                word = int(words[kb, n, h])
+                for g in range(8):
+                    base = 64 * kb + _group_dense_offset(g, h)
+                    nib = (word >> (4 * g)) & 15
+                    out[n, base + (nib & 3)] = wc[kb, n, 16 * h + 2 * g]
+                    out[n, base + (nib >> 2)] = wc[kb, n, 16 * h + 2 * g + 1]
+    return out
+
+
+def sparse24_int8_linear(x: torch.Tensor, weight: torch.Tensor, bias) -> torch.Tensor:
+    """Dynamic int8 Linear whose float weight is first magnitude-pruned to 2:4
+    (sparse.py:6-25), then quantised per output channel: the combination the
+    benchmark's int8 + 2:4 MLP configuration uses."""
+    return dynamic_int8_linear(x, prune_2_of_4(weight), bias)

@@ -18,9 +18,11 @@ from .build_sam import (
 )
 from .predictor import SamPredictor
 from .quant import Int8DynamicLinear, apply_dynamic_quant
+from .sparse import Int8Sparse24Linear, apply_fake_sparsity, apply_sparse
 
 __all__ = [
     "build_sam", "build_sam_vit_h", "build_sam_vit_l", "build_sam_vit_b", "sam_model_registry",
     "build_sam_fast", "build_sam_fast_vit_h", "build_sam_fast_vit_l", "build_sam_fast_vit_b",
     "sam_model_fast_registry", "SamPredictor", "Int8DynamicLinear", "apply_dynamic_quant",
+    "Int8Sparse24Linear", "apply_fake_sparsity", "apply_sparse",
 ]

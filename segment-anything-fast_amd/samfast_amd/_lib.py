@@ -34,6 +34,11 @@ _SIGNATURES = {
     "samfast_gemm_i8_fused": (
         _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _i32,
                _ptr, _i64, _ptr, _ptr]),
+    "samfast_prune24_pack_i8": (_i32, [_ptr, _ptr, _ptr, _i32, _i32, _ptr]),
+    "samfast_gemm_i8_sparse24_i32": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _i32, _i32, _ptr]),
+    "samfast_gemm_i8_sparse24_fused": (
+        _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _i32,
+               _ptr, _i64, _ptr]),
 }
 
 EPILOGUE_NONE, EPILOGUE_GELU, EPILOGUE_RESIDUAL = 0, 1, 2

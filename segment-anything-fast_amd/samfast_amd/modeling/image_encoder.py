@@ -118,12 +118,14 @@ class Block(nn.Module):
         self.window_size = window_size
 
     def _int8_fused_ok(self, x: torch.Tensor) -> bool:
-        from ..quant import Int8DynamicLinear
+        from ..quant import Int8LinearBase
         attn, mlp = self.attn, self.mlp
         if not (FUSED_BLOCK and flash_4.USE_CUSTOM_KERNEL and x.is_cuda
                 and x.dtype == torch.bfloat16 and x.dim() == 4 and attn.use_rel_pos):
             return False
-        if not all(isinstance(m, Int8DynamicLinear) for m in (attn.qkv, attn.proj, mlp.lin1, mlp.lin2)):
+        if not all(isinstance(m, Int8LinearBase) for m in (attn.qkv, attn.proj, mlp.lin1, mlp.lin2)):
+            return False
+        if self.window_size > 0 and not attn.proj.supports_row_scatter:
             return False
         if not (isinstance(self.norm1, nn.LayerNorm) and isinstance(self.norm2, nn.LayerNorm)
                 and self.norm1.elementwise_affine and self.norm2.elementwise_affine
@@ -155,20 +157,18 @@ class Block(nn.Module):
         # norm1 (+ window partition with zero padding) + qkv's activation quantiser
         xq, sx = ops.layernorm_quant(tokens, self.norm1.weight, self.norm1.bias, self.norm1.eps, row_map)
         Bw = xq.shape[0] // N
-        qkv = ops.gemm_i8_fused(xq, sx, attn.qkv.wq, attn.qkv.sw, attn.qkv.bias_f32, _lib.EPILOGUE_NONE)
+        qkv = attn.qkv.linear_fused(xq, sx, _lib.EPILOGUE_NONE)
         qkv = qkv.view(Bw, N, 3, nH, hd)
         q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
         o = ops.attn_relpos(q, k, v, attn.rel_pos_h, attn.rel_pos_w, (gh, gw), attn.scale)
         oq, so = ops.quant_rowwise(o.permute(0, 2, 1, 3).reshape(Bw * N, C))
         # proj + window unpartition + `shortcut + x`
-        tokens = ops.gemm_i8_fused(oq, so, attn.proj.wq, attn.proj.sw, attn.proj.bias_f32,
-                                   _lib.EPILOGUE_RESIDUAL, residual=tokens, dst_row=row_map)
+        tokens = attn.proj.linear_fused(oq, so, _lib.EPILOGUE_RESIDUAL, residual=tokens, dst_row=row_map)
         # norm2 + lin1's quantiser, lin1 + GELU, lin2's quantiser, lin2 + `x + mlp(...)`
         hq, sh = ops.layernorm_quant(tokens, self.norm2.weight, self.norm2.bias, self.norm2.eps)
-        h = ops.gemm_i8_fused(hq, sh, mlp.lin1.wq, mlp.lin1.sw, mlp.lin1.bias_f32, _lib.EPILOGUE_GELU)
+        h = mlp.lin1.linear_fused(hq, sh, _lib.EPILOGUE_GELU)
         gq, sg = ops.quant_rowwise(h)
-        tokens = ops.gemm_i8_fused(gq, sg, mlp.lin2.wq, mlp.lin2.sw, mlp.lin2.bias_f32,
-                                   _lib.EPILOGUE_RESIDUAL, residual=tokens, out=tokens)
+        tokens = mlp.lin2.linear_fused(gq, sg, _lib.EPILOGUE_RESIDUAL, residual=tokens, out=tokens)
         return tokens.view(B, H, W, C)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:

@@ -289,6 +289,86 @@ def gemm_i8_fused(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torc
     return out
 
 
+def prune24_pack(wq: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """int8 (N, K) -> packed 2:4 form (wc int8 (K/64, N, 32), widx int32 (K/64, N, 2)): per
+    aligned group of 4 along K the two largest magnitudes are kept (ties: lowest position).
+    Lossless for a matrix that already is 2:4.  Layout: include/samfast.h."""
+    _require_gpu(wq)
+    if wq.dtype != torch.int8 or wq.dim() != 2 or not wq.is_contiguous():
+        raise RuntimeError("samfast: prune24_pack needs a contiguous int8 (N, K) tensor")
+    N, K = wq.shape
+    if K % 64 != 0:
+        raise RuntimeError("samfast: prune24_pack needs K % 64 == 0")
+    wc = torch.empty((K // 64, N, 32), dtype=torch.int8, device=wq.device)
+    widx = torch.empty((K // 64, N, 2), dtype=torch.int32, device=wq.device)
+    code = _lib.load().samfast_prune24_pack_i8(wq.data_ptr(), wc.data_ptr(), widx.data_ptr(), N, K,
+                                               _stream())
+    _lib.check(code, "prune24_pack_i8")
+    return wc, widx
+
+
+def _check_sparse24(xq: torch.Tensor, wc: torch.Tensor, widx: torch.Tensor) -> Tuple[int, int, int]:
+    if xq.dtype != torch.int8 or xq.dim() != 2 or not xq.is_contiguous():
+        raise RuntimeError("samfast: sparse24 GEMM needs a contiguous int8 (M, K) activation")
+    M, K = xq.shape
+    if (wc.dtype != torch.int8 or widx.dtype != torch.int32 or wc.dim() != 3 or widx.dim() != 3
+            or not (wc.is_contiguous() and widx.is_contiguous())
+            or wc.shape[0] * 64 != K or wc.shape[2] != 32
+            or tuple(widx.shape) != (wc.shape[0], wc.shape[1], 2)):
+        raise RuntimeError("samfast: packed weight must be int8 (K/64, N, 32) + int32 (K/64, N, 2)")
+    return M, wc.shape[1], K
+
+
+def gemm_i8_sparse24_i32(xq: torch.Tensor, wc: torch.Tensor, widx: torch.Tensor) -> torch.Tensor:
+    """int8 (M, K) x packed 2:4 int8 weight -> int32 (M, N), exact."""
+    _require_gpu(xq, wc, widx)
+    M, N, K = _check_sparse24(xq, wc, widx)
+    acc = torch.empty((M, N), dtype=torch.int32, device=xq.device)
+    lib = _lib.load()
+    code = _timed(
+        "gemm_i8_sp24_i32", 1.0 * M * N * K, "op",
+        lambda: lib.samfast_gemm_i8_sparse24_i32(xq.data_ptr(), wc.data_ptr(), widx.data_ptr(),
+                                                 acc.data_ptr(), M, N, K, _stream()))
+    _lib.check(code, "gemm_i8_sparse24_i32")
+    return acc
+
+
+def gemm_i8_sparse24_fused(xq: torch.Tensor, sx: torch.Tensor, wc: torch.Tensor, widx: torch.Tensor,
+                           sw: torch.Tensor, bias: Optional[torch.Tensor], epilogue: int,
+                           residual: Optional[torch.Tensor] = None,
+                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """gemm_i8_fused (no row scatter) with the weight in the packed 2:4 form.  The work
+    reported to record_launches is the multiply-adds the sparse matrix cores execute
+    (half the dense count)."""
+    _require_gpu(xq, sx, wc, widx, sw, bias, residual)
+    M, N, K = _check_sparse24(xq, wc, widx)
+    if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != M or sw.numel() != N:
+        raise RuntimeError("samfast: scales must be fp32 of length M and N")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N):
+        raise RuntimeError("samfast: bias must be fp32 of length N")
+    if epilogue == _lib.EPILOGUE_RESIDUAL:
+        if residual is None or tuple(residual.shape) != (M, N) or residual.stride(1) != 1 \
+                or residual.dtype != torch.bfloat16:
+            raise RuntimeError("samfast: residual must be a bf16 (M, N) tensor")
+        if out is None:
+            out = torch.empty_like(residual)
+    elif out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=xq.device)
+    lib = _lib.load()
+    name = {_lib.EPILOGUE_NONE: "gemm_i8_sp24_scale_bias", _lib.EPILOGUE_GELU: "gemm_i8_sp24_gelu",
+            _lib.EPILOGUE_RESIDUAL: "gemm_i8_sp24_residual"}.get(epilogue, "gemm_i8_sp24_fused")
+    code = _timed(
+        name, 1.0 * M * N * K, "op",
+        lambda: lib.samfast_gemm_i8_sparse24_fused(
+            xq.data_ptr(), sx.data_ptr(), wc.data_ptr(), widx.data_ptr(), sw.data_ptr(),
+            bias.data_ptr() if bias is not None else None, out.data_ptr(), out.stride(0),
+            M, N, K, _lib.SAMFAST_BF16, int(epilogue),
+            residual.data_ptr() if residual is not None else None,
+            residual.stride(0) if residual is not None else 0, _stream()))
+    _lib.check(code, "gemm_i8_sparse24_fused")
+    return out
+
+
 _window_maps = {}
 
 

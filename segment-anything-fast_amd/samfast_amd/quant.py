@@ -23,6 +23,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
+from ._lib import EPILOGUE_NONE
 from .tools import replace_with_custom_fn_if_matches_filter
 
 
@@ -36,17 +37,20 @@ def quantize_weight_per_channel(weight: torch.Tensor):
     return q.contiguous(), scale.contiguous()
 
 
-class Int8DynamicLinear(nn.Module):
-    """Scales and the fp32 bias are registered as int32 bit patterns so that a
+class Int8LinearBase(nn.Module):
+    """What every int8 Linear here shares: shapes, per-channel weight scales and bias.
+
+    Scales and the fp32 bias are registered as int32 bit patterns so that a
     later `model.to(torch.bfloat16)` (which casts every floating-point buffer)
     cannot round them; they are viewed back as fp32 at call time."""
 
-    def __init__(self, in_features: int, out_features: int, wq: torch.Tensor, sw: torch.Tensor,
+    supports_row_scatter = True  # linear_fused accepts dst_row
+
+    def __init__(self, in_features: int, out_features: int, sw: torch.Tensor,
                  bias: Optional[torch.Tensor]) -> None:
         super().__init__()
         self.in_features = in_features
         self.out_features = out_features
-        self.register_buffer("wq", wq)
         self.register_buffer("sw_bits", sw.to(torch.float32).contiguous().view(torch.int32))
         if bias is not None:
             self.bias = nn.Parameter(bias.detach().clone(), requires_grad=False)
@@ -55,11 +59,6 @@ class Int8DynamicLinear(nn.Module):
         else:
             self.bias = None
             self.bias_bits = None
-
-    @classmethod
-    def from_float(cls, linear: nn.Linear) -> "Int8DynamicLinear":
-        wq, sw = quantize_weight_per_channel(linear.weight)
-        return cls(linear.in_features, linear.out_features, wq, sw, linear.bias)
 
     @property
     def sw(self) -> torch.Tensor:
@@ -73,14 +72,38 @@ class Int8DynamicLinear(nn.Module):
     def weight(self) -> torch.Tensor:
         return self.wq.to(torch.float32) * self.sw[:, None]
 
+    def linear_fused(self, xq, sx, epilogue, residual=None, dst_row=None, out=None):
+        raise NotImplementedError
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         lead = x.shape[:-1]
         x2 = x.reshape(-1, self.in_features)
         if x2.dtype != torch.bfloat16:
             x2 = x2.to(torch.bfloat16)
         xq, sx = ops.quant_rowwise(x2)
-        y = ops.gemm_i8_scale_bias(xq, sx, self.wq, self.sw, self.bias_f32)
+        y = self.linear_fused(xq, sx, EPILOGUE_NONE)
         return y.reshape(*lead, self.out_features)
+
+
+class Int8DynamicLinear(Int8LinearBase):
+    """Dense int8 weight `wq` (N, K)."""
+
+    def __init__(self, in_features: int, out_features: int, wq: torch.Tensor, sw: torch.Tensor,
+                 bias: Optional[torch.Tensor]) -> None:
+        super().__init__(in_features, out_features, sw, bias)
+        self.register_buffer("wq", wq)
+
+    @classmethod
+    def from_float(cls, linear: nn.Linear) -> "Int8DynamicLinear":
+        wq, sw = quantize_weight_per_channel(linear.weight)
+        return cls(linear.in_features, linear.out_features, wq, sw, linear.bias)
+
+    def linear_fused(self, xq: torch.Tensor, sx: torch.Tensor, epilogue: int,
+                     residual: Optional[torch.Tensor] = None, dst_row: Optional[torch.Tensor] = None,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The GEMM + epilogue on already quantised rows (see ops.gemm_i8_fused)."""
+        return ops.gemm_i8_fused(xq, sx, self.wq, self.sw, self.bias_f32, epilogue,
+                                 residual=residual, dst_row=dst_row, out=out)
 
     def extra_repr(self) -> str:
         return f"in_features={self.in_features}, out_features={self.out_features}, int8 dynamic"
