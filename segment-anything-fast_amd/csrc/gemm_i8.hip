@@ -163,6 +163,103 @@ SF_DEVICE void gemm_epilogue(const GemmArgs& a, i32x16 (&acc)[TM][4], int m0, in
   }
 }
 
+// Staged epilogue of the main kernel (TM = 2, bf16 outputs).  Phase 1: every lane scales
+// its accumulators (row scales, column scales and bias come from a small LDS area that was
+// filled by global->LDS loads at kernel start) and writes the bf16 results into the LDS
+// that held the operand stages, as a row-major 128 x 256 tile.  Phase 2: the workgroup
+// walks that tile 8 rows at a time, 16 bytes per lane, so that every global store (and
+// residual load) instruction covers two whole 512-byte row segments.
+constexpr int EP_STRIDE = 544;                 // tile row pitch in bytes: rows r and r+4 half a bank cycle apart
+constexpr int EP_SCALE_BYTES = 512 + 1024 + 1024;  // sx[128], sw[256], bias[256] as fp32
+constexpr int EP_ROWMAP_BYTES = 512;                // dst_row[128] (EPI_RESIDUAL)
+constexpr int EP_PAD_BYTES = 256;                   // landing pad of the residual prefetch
+
+template <int EPI>
+SF_DEVICE void gemm_epilogue_staged(const GemmArgs& a, i32x16 (&acc)[2][4], unsigned char* lds,
+                                    const unsigned char* sc, int m0, int n0, int wm, int wn,
+                                    int lr, int lh, int tid) {
+  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt 0, lgkmcnt 0
+  __builtin_amdgcn_s_barrier();        // nobody reads operand stages any more
+  __builtin_amdgcn_sched_barrier(0);
+
+  // phase-2 geometry: pass p (0..15) handles tile row 8p + rsub, 16-byte chunk `chunk`
+  const int chunk = tid & 31, rsub = tid >> 5;
+  const int n = n0 + chunk * 8;
+  const bool col_ok = n < a.N;  // N % 8 == 0
+  auto out_row = [&](int p) {
+    const int row = 8 * p + rsub;
+    if (m0 + row >= a.M || !col_ok) return -1;
+    if (EPI == EPI_RESIDUAL_BF16 && a.dst_row)  // the row map of this tile sits behind the scales
+      return *reinterpret_cast<const int*>(sc + EP_SCALE_BYTES + row * 4);
+    return m0 + row;
+  };
+  // EPI_RESIDUAL: the residual values are requested before the conversion work below, so
+  // their latency is hidden behind it
+  u32x4 res[16];
+  if (EPI == EPI_RESIDUAL_BF16) {
+#pragma unroll
+    for (int p = 0; p < 16; ++p) {
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      res[p] = z;
+      const int dr = out_row(p);
+      if (dr >= 0) res[p] = *reinterpret_cast<const u32x4*>(a.residual + (int64_t)dr * a.ld_res + n);
+    }
+  }
+
+  {
+    const f32x4 swv = *reinterpret_cast<const f32x4*>(sc + 512 + (wn * 128 + 4 * lr) * 4);
+    f32x4 bv4 = {0.f, 0.f, 0.f, 0.f};
+    if (a.bias) bv4 = *reinterpret_cast<const f32x4*>(sc + 1536 + (wn * 128 + 4 * lr) * 4);
+    unsigned char* dst = lds + (wm * 64 + 4 * lh) * EP_STRIDE + (wn * 128 + 4 * lr) * 2;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      f32x4 sxv[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        sxv[g] = *reinterpret_cast<const f32x4*>(sc + (wm * 64 + i * 32 + 8 * g + 4 * lh) * 4);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float s = sxv[r >> 2][r & 3];
+        float y[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          // three separately rounded fp32 operations (no fused multiply-add)
+          float t = (float)acc[i][j][r] * s;
+          t = t * swv[j];
+          y[j] = t + bv4[j];
+        }
+        u32x2 o = {pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3])};
+        if (EPI == EPI_GELU_BF16) {
+          // activation of the bf16-rounded Linear output, as a separate GELU would see it
+          o[0] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[0])), gelu_erf(bf16_hi_to_f32(o[0])));
+          o[1] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[1])), gelu_erf(bf16_hi_to_f32(o[1])));
+        }
+        *reinterpret_cast<u32x2*>(dst + (i * 32 + 8 * (r >> 2) + (r & 3)) * EP_STRIDE) = o;
+      }
+    }
+  }
+  // LDS writes done and, once for all of phase 2, the residual values have arrived: later
+  // vmcnt waits would also wait for the stores issued in between
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+
+  unsigned short* outp = reinterpret_cast<unsigned short*>(a.out);
+#pragma unroll
+  for (int p = 0; p < 16; ++p) {
+    const int dr = out_row(p);
+    u32x4 val = *reinterpret_cast<const u32x4*>(lds + (8 * p + rsub) * EP_STRIDE + chunk * 16);
+    if (EPI == EPI_RESIDUAL_BF16) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        // bf16 add of the bf16-rounded Linear output and the residual stream
+        val[c] = pack_bf16x2(bf16_lo_to_f32(val[c]) + bf16_lo_to_f32(res[p][c]),
+                             bf16_hi_to_f32(val[c]) + bf16_hi_to_f32(res[p][c]));
+    }
+    if (dr >= 0) *reinterpret_cast<u32x4*>(outp + (int64_t)dr * a.ldo + n) = val;
+  }
+}
+
 // 16-byte chunk c of LDS row r lives at chunk position c ^ lds_swizzle(r).  With it the
 // operand reads (one chunk of 8 / 16 consecutive rows per LDS cycle) and the tile writes
 // (4 chunks of 2 / 4 consecutive rows per cycle) both touch every bank once, whether the
@@ -174,7 +271,9 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
   constexpr int GBM = 64 * TM;
   constexpr int GSTAGE = (GBM + GBN) * GLD;
   constexpr int NST = GENERIC ? 2 : (TM == 4 ? 4 : 3);  // LDS stages
-  __shared__ __attribute__((aligned(16))) unsigned char lds[NST * GSTAGE];
+  constexpr bool STAGED = !GENERIC && TM == 2 && EPI != EPI_I32;  // epilogue through LDS
+  static_assert(!STAGED || 128 * EP_STRIDE <= NST * GSTAGE, "output tile must fit in the operand stages");
+  __shared__ __attribute__((aligned(16))) unsigned char lds[NST * GSTAGE + (STAGED ? EP_SCALE_BYTES + EP_ROWMAP_BYTES + EP_PAD_BYTES : 0)];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -353,6 +452,20 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
     auto wait_imm = [](int n) constexpr { return 0x0070 | (n & 15) | ((n >> 4) << 14); };
     static_assert((NST - 1) * NLD <= 63, "vmcnt immediate");
 
+    if constexpr (STAGED) {
+      // row scales, column scales and bias of this tile, 4 bytes per lane, straight into LDS;
+      // they are the oldest loads in flight, so every later vmcnt wait covers them
+      unsigned char* sc = lds + NST * GSTAGE;
+      const int mm = min(m0 + (wave_u & 1) * 64 + lane, a.M - 1);
+      const int nn = min(n0 + wave_u * 64 + lane, a.N - 1);
+      __builtin_amdgcn_global_load_lds((gptr_t)(a.sx + mm), (lptr_t)(sc + (wave_u & 1) * 256), 4, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(a.sw + nn), (lptr_t)(sc + 512 + wave_u * 256), 4, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)((a.bias ? a.bias : a.sw) + nn),
+                                       (lptr_t)(sc + 1536 + wave_u * 256), 4, 0, 0);
+      if (EPI == EPI_RESIDUAL_BF16 && a.dst_row)  // uniform: every wave issues it or none does
+        __builtin_amdgcn_global_load_lds((gptr_t)(a.dst_row + mm),
+                                         (lptr_t)(sc + EP_SCALE_BYTES + (wave_u & 1) * 256), 4, 0, 0);
+    }
     int st[NST];  // st[j] = LDS offset of the stage holding tile kt + j (uniform, rotated)
 #pragma unroll
     for (int j = 0; j < NST; ++j) {
@@ -367,10 +480,11 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
     // ISSUE: fetch tile kt+NST into the stage freed at the barrier; NEXT: a tile kt+1
     // exists; KEEP: tiles that may stay in flight across the barrier (after tile kt+1).
     // (sched_group_barrier masks: 0x008 MFMA, 0x100 LDS read, 0x020 global read)
-    auto iteration = [&](int kt, auto issue_c, auto next_c, auto keep_c) {
+    auto iteration = [&](int kt, auto issue_c, auto next_c, auto keep_c, auto extra_c) {
       constexpr bool ISSUE = decltype(issue_c)::value != 0;
       constexpr bool NEXT = decltype(next_c)::value != 0;
       constexpr int KEEP = decltype(keep_c)::value;
+      constexpr int EXTRA = decltype(extra_c)::value;  // younger non-tile loads that may stay in flight
       frags_at(st[0], 1, fa1, fb1);
       mma(fa0, fb0);
 #pragma unroll
@@ -380,7 +494,7 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
       }
       __builtin_amdgcn_sched_barrier(0);
       // own LDS reads of this stage done; own share of tile kt+1 landed; then all waves meet
-      __builtin_amdgcn_s_waitcnt(wait_imm(KEEP * NLD));
+      __builtin_amdgcn_s_waitcnt(wait_imm(NEXT ? KEEP * NLD + EXTRA : 63));
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (ISSUE) dma_issue(kt + NST, st[0]);
@@ -400,15 +514,35 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
     };
     using Yes = std::integral_constant<int, 1>;
     using No = std::integral_constant<int, 0>;
-    for (; kt + NST < nk; ++kt) iteration(kt, Yes{}, Yes{}, std::integral_constant<int, NST - 2>{});
+    for (; kt + NST < nk; ++kt) iteration(kt, Yes{}, Yes{}, std::integral_constant<int, NST - 2>{}, No{});
+    // The residual rows of this tile are touched now (one dword per 128-byte line, landing in
+    // an unused LDS pad), so that the epilogue's residual loads find them in L2.
+    constexpr int NPF = (STAGED && EPI == EPI_RESIDUAL_BF16) ? 2 : 0;
+    if constexpr (NPF > 0) {
+      const unsigned char* sc = lds + NST * GSTAGE;
+#pragma unroll
+      for (int i = 0; i < NPF; ++i) {
+        const int line = (wave_u * NPF + i) * 64 + lane;  // 512 lines: 128 rows x 4
+        const int row = min(line >> 2, a.M - 1 - m0);
+        int dr = m0 + row;
+        if (a.dst_row) dr = max(*reinterpret_cast<const int*>(sc + EP_SCALE_BYTES + row * 4), 0);
+        const int col = min(n0 + (line & 3) * 64, a.N - 8);
+        __builtin_amdgcn_global_load_lds((gptr_t)(a.residual + (int64_t)dr * a.ld_res + col),
+                                         (lptr_t)(lds + NST * GSTAGE + EP_SCALE_BYTES + EP_ROWMAP_BYTES), 4, 0, 0);
+      }
+    }
+    using Extra = std::integral_constant<int, NPF>;
     // the last NST iterations fetch nothing; fewer and fewer tiles remain in flight
-    if constexpr (NST == 4) iteration(kt++, No{}, Yes{}, std::integral_constant<int, 2>{});
-    iteration(kt++, No{}, Yes{}, std::integral_constant<int, 1>{});
-    iteration(kt++, No{}, Yes{}, No{});
-    iteration(kt++, No{}, No{}, No{});
+    if constexpr (NST == 4) iteration(kt++, No{}, Yes{}, std::integral_constant<int, 2>{}, Extra{});
+    iteration(kt++, No{}, Yes{}, std::integral_constant<int, 1>{}, Extra{});
+    iteration(kt++, No{}, Yes{}, No{}, Extra{});
+    iteration(kt++, No{}, No{}, No{}, Extra{});
   }
 
-  gemm_epilogue<EPI, TM>(a, acc, m0, n0, wm, wn, lr, lh);
+  if constexpr (STAGED)
+    gemm_epilogue_staged<EPI>(a, acc, lds, lds + NST * GSTAGE, m0, n0, wm, wn, lr, lh, tid);
+  else
+    gemm_epilogue<EPI, TM>(a, acc, m0, n0, wm, wn, lr, lh);
 }
 
 static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t* wq,
@@ -428,8 +562,7 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
     SF_REQUIRE(aligned16(out) && ldo % 4 == 0, "gemm_i8: int32 output must be 16-byte aligned rows");
   } else {
     SF_REQUIRE(sx && sw, "gemm_i8: null scale pointer");
-    SF_REQUIRE((reinterpret_cast<uintptr_t>(out) & 7u) == 0 && ldo % 4 == 0,
-               "gemm_i8: bf16 output rows must be 8-byte aligned");
+    SF_REQUIRE(aligned16(out) && ldo % 8 == 0, "gemm_i8: bf16 output rows must be 16-byte aligned");
     SF_REQUIRE(aligned16(sw) && aligned16(sx) && (!bias || aligned16(bias)),
                "gemm_i8: sx / sw / bias must be 16-byte aligned");
   }
@@ -440,9 +573,8 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   a.residual = reinterpret_cast<const unsigned short*>(residual);
   a.ld_res = ld_res; a.dst_row = dst_row;
   if (epi == EPI_RESIDUAL_BF16) {
-    SF_REQUIRE(residual && (reinterpret_cast<uintptr_t>(residual) & 7u) == 0 && ld_res >= N &&
-                   ld_res % 4 == 0,
-               "gemm_i8: residual must be non-null with 8-byte aligned rows");
+    SF_REQUIRE(residual && aligned16(residual) && ld_res >= N && ld_res % 8 == 0,
+               "gemm_i8: residual must be non-null with 16-byte aligned rows");
     SF_REQUIRE(!dst_row || aligned16(dst_row), "gemm_i8: dst_row must be 16-byte aligned");
   }
   const char* force = getenv("SAMFAST_GEMM_TM");  // tuning aid: 2 or 4
