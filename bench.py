@@ -29,13 +29,13 @@ PEAK = {"op": ("mfma", 5.0e15, "TOP/s"),       # int8 dense MFMA
         "flop": ("mfma", 2.5e15, "TFLOP/s"),   # bf16 dense MFMA
         "byte": ("hbm", 8.0e12, "GB/s")}       # HBM3E
 
-# HBM-side bytes per launch (average over the launches of one encoder step) from the two
-# `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this script summarised in
-# profiles/bench_vit_h_bs16_pmc_traffic.txt, each counter scaled by what it reads for the
-# 1 GiB --calibration-copy dispatch (FETCH_SIZE x 1.5957, WRITE_SIZE x 1.0).  Valid for the
-# default workload (vit_h, batch 16) only.
-TRAFFIC = {"gemm_i8_kernel": 1.1377e9, "attn_window": 1.0784e9, "attn_global": 6.951e8,
-           "quant_rowwise": 3.951e8}
+# Bytes per launch that cross the L2 <-> fabric boundary (average over the launches of one
+# encoder step), from the two `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this
+# script summarised in profiles/bench_vit_h_bs16_pmc_traffic.txt, each counter scaled by what
+# it reads for the 1 GiB --calibration-copy dispatch (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
+# Valid for the default workload (vit_h, batch 16, dense int8 linears) only.
+TRAFFIC = {"gemm_i8_kernel": 1.2747e9, "attn_window": 1.2872e9, "attn_global": 8.182e8,
+           "quant_rowwise": 6.515e8, "layernorm_quant": 2.607e8}
 
 
 def parse():
@@ -48,6 +48,9 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-gpu-baseline", action="store_true")
     p.add_argument("--bf16-linears", action="store_true", help="keep nn.Linear (attention kernels only)")
+    p.add_argument("--sparse-mlp", action="store_true",
+                   help="lin1 / lin2 magnitude-pruned 2:4 on the sparse int8 matrix cores (the int8 + 2:4 "
+                        "configuration); every other Linear dense int8")
     p.add_argument("--calibration-copy", action="store_true",
                    help="also run one 1 GiB device-to-device copy (a known-size reference for "
                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -90,7 +93,8 @@ def main():
         sys.exit(2)
 
     import torch
-    from samfast_amd import apply_dynamic_quant, flash_4, ops
+    from samfast_amd import apply_dynamic_quant, apply_sparse, flash_4, ops
+    from samfast_amd.sparse import mlp_only
     from samfast_amd.build_sam import build_image_encoder
     from samfast_amd.synthetic import init_encoder_weights, make_images
 
@@ -103,6 +107,8 @@ def main():
     enc = build_image_encoder(args.model)
     sd_fp32 = {k: v.clone() for k, v in init_encoder_weights(enc, seed=0).items()}
     enc = enc.eval().to(torch.bfloat16).to(dev)
+    if args.sparse_mlp:
+        apply_sparse(enc, mlp_only)
     if not args.bf16_linears:
         apply_dynamic_quant(enc)
     images = make_images(args.batch, seed=1).to(torch.bfloat16).to(dev)
@@ -129,7 +135,8 @@ def main():
     # the dominant kernel: every epilogue variant of gemm_i8_kernel counts as one kernel
     fam = {}
     for name, d in summary.items():
-        key = "gemm_i8_kernel" if name.startswith("gemm_i8") else name
+        key = ("gemm_i8_sp24_kernel" if name.startswith("gemm_i8_sp24") else
+               "gemm_i8_kernel" if name.startswith("gemm_i8") else name)
         f = fam.setdefault(key, dict(launches=0, work=0.0, unit=d["unit"], ms=0.0))
         f["launches"] += d["launches"]
         f["work"] += d["work"]
@@ -139,20 +146,25 @@ def main():
     dk = families[dominant]
     roofline = {"kernel": dominant, "bound": dk["bound"], "achieved": dk["achieved"],
                 "peak": dk["peak"], "unit": dk["unit"], "frac": dk["frac"],
-                "traffic": TRAFFIC.get(dominant) if (args.model, args.batch) == ("vit_h", 16) else None,
+                "traffic": TRAFFIC.get(dominant)
+                if (args.model, args.batch, args.sparse_mlp) == ("vit_h", 16, False) else None,
                 "avg_us": dk["avg_us"], "launches_per_step": dk["launches"],
                 "ms_per_step": dk["ms_total"]}
 
     result = {
-        "metric": "images/s ViT-H encoder bs16 1024^2" if (args.model, args.batch) == ("vit_h", 16)
-        else f"images/s {args.model} encoder bs{args.batch} 1024^2",
+        "metric": ("images/s ViT-H encoder bs16 1024^2" if (args.model, args.batch) == ("vit_h", 16)
+                   else f"images/s {args.model} encoder bs{args.batch} 1024^2")
+        + (" (2:4 sparse MLP)" if args.sparse_mlp else ""),
         "value": round(args.batch / sec, 3), "unit": "images/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 attention + int8 linears (int32 accumulate)" if not args.bf16_linears else "bf16",
+        "dtype": ("bf16" if args.bf16_linears and not args.sparse_mlp else
+                  "bf16 attention + int8 linears (int32 accumulate)"
+                  + (", lin1/lin2 2:4 sparse" if args.sparse_mlp else "")),
         "data": "synthetic (seeded uniform images, random-init weights)",
         "config": {"workload": f"SAM {args.model} image encoder forward, batch {args.batch}, "
-                               "1024x1024, rel-pos attention + dynamic int8 linears",
+                               "1024x1024, rel-pos attention + dynamic int8 linears"
+                               + (" (lin1 / lin2 pruned 2:4, sparse int8 MFMA)" if args.sparse_mlp else ""),
                    "batch": args.batch, "image": 1024},
         "output_finite": finite,
         "roofline": roofline,
@@ -164,6 +176,9 @@ def main():
         base = build_image_encoder(args.model)
         base.load_state_dict(sd_fp32)
         base = base.eval().to(torch.bfloat16).to(dev)
+        if args.sparse_mlp:  # same pruned weights, dense bf16 kernels
+            from samfast_amd import apply_fake_sparsity
+            apply_fake_sparsity(base, mlp_only)
         flash_4.USE_CUSTOM_KERNEL = False
         try:
             with torch.no_grad():
