@@ -110,3 +110,24 @@ def test_prune_2_of_4_bruteforce_and_library():
     sp.step()
     sp.squash_mask()
     assert torch.equal(lin.weight.detach(), p)
+
+
+def test_pack_2_of_4_round_trip_and_invariants():
+    """The packed 2:4 form stands for exactly the magnitude-pruned matrix; positions are
+    ordered and every group keeps two entries.  (Which stored byte the hardware pairs with
+    which dense k is fixed by the GPU bit-exact tests, not here.)"""
+    rng = np.random.default_rng(11)
+    for hi in (128, 3):  # full range, and a range that forces ties and zeros
+        wq = rng.integers(-hi + 1, hi, size=(6, 192), dtype=np.int8)
+        wc, widx = orq.pack_2_of_4(wq)
+        assert wc.shape == (3, 6, 32) and widx.shape == (3, 6, 2) and widx.dtype == np.int32
+        dense = orq.unpack_2_of_4(wc, widx)
+        pruned = orq.prune_2_of_4(torch.from_numpy(wq.astype(np.float32))).numpy().astype(np.int8)
+        assert np.array_equal(dense, pruned)
+        words = widx.view(np.uint32)
+        for g in range(8):
+            nib = (words >> (4 * g)) & 15
+            assert np.all((nib & 3) < (nib >> 2))
+        # a matrix that already is 2:4 is packed without loss
+        wc2, widx2 = orq.pack_2_of_4(pruned)
+        assert np.array_equal(orq.unpack_2_of_4(wc2, widx2), pruned)
