@@ -39,6 +39,17 @@ extern "C" {
 #define SAMFAST_E_UNSUPPORTED (-2)  /* a shape or type no kernel here covers */
 #define SAMFAST_E_LAUNCH (-3)       /* the HIP runtime refused the launch */
 
+/*
+ * Layouts of an int8 GEMM operand with R rows and K columns (activations xq: R = M; dense
+ * weights wq: R = N):
+ *   ROWMAJOR  (R, K), element (r, k) at r*K + k - what torch._int_mm takes;
+ *   KB64      K-block major, (K/64, R, 64): element (r, k) at ((k/64)*R + r)*64 + k%64, so the
+ *             64-byte k tile of consecutive rows is contiguous memory and the GEMM reads whole
+ *             cache lines.  K % 64 == 0.  The quantisers can write it, the fused GEMMs read it.
+ */
+#define SAMFAST_LAYOUT_ROWMAJOR 0
+#define SAMFAST_LAYOUT_KB64 1
+
 int samfast_version(void);
 /* "gfx950" - the only architecture the code objects are built for */
 const char* samfast_arch(void);
@@ -101,10 +112,11 @@ int samfast_attn_relpos_bias_fwd(
  * Writes xq (M, K) int8 contiguous and sx (M) fp32.  Stands for the per-token
  * activation quantiser torchao.apply_dynamic_quant installs in front of every
  * Linear (call site experiments/eval_combo.py:357-359).  K % 8 == 0, K <= 8192.
+ * `layout` is the layout xq is written in (SAMFAST_LAYOUT_*).
  */
 int samfast_quant_rowwise_i8(
     const void* x, int64_t ldx, int8_t* xq, float* sx,
-    int64_t M, int K, int dtype, void* stream);
+    int64_t M, int K, int dtype, int layout, void* stream);
 
 /*
  * acc[m, n] = sum_k xq[m, k] * wq[n, k], int32, exact.  xq (M, K) and wq (N, K)
@@ -141,7 +153,7 @@ int samfast_gemm_i8_scale_bias(
 int samfast_layernorm_quant_i8(
     const void* x, int64_t ldx, const void* gamma, const void* beta, float eps,
     const int32_t* src_row, int8_t* xq, float* sx,
-    int64_t M, int K, int dtype, void* stream);
+    int64_t M, int K, int dtype, int layout, void* stream);
 
 /* epilogues of samfast_gemm_i8_fused */
 #define SAMFAST_EPILOGUE_NONE 0      /* same as samfast_gemm_i8_scale_bias */
@@ -158,12 +170,13 @@ int samfast_layernorm_quant_i8(
  *             map this is proj + window_unpartition + `shortcut + x`
  *             (modeling/image_encoder.py:176-180); with the identity map it is lin2 +
  *             `x + mlp(...)` (:181).  y and residual may be the same buffer.
+ * `layout` names the layout of BOTH xq and wq (SAMFAST_LAYOUT_*).
  */
 int samfast_gemm_i8_fused(
     const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
     const float* bias, void* y, int64_t ldy,
     int64_t M, int N, int K, int dtype, int epilogue,
-    const void* residual, int64_t ld_res, const int32_t* dst_row, void* stream);
+    const void* residual, int64_t ld_res, const int32_t* dst_row, int layout, void* stream);
 
 /*
  * 2:4-sparse weights for the sparse int8 matrix cores (v_smfmac_i32_32x32x64_i8).
@@ -195,13 +208,14 @@ int samfast_gemm_i8_sparse24_i32(
  * samfast_gemm_i8_fused (epilogues NONE / GELU / RESIDUAL, no row scatter) with the weight
  * in the packed 2:4 form: the semi-structured Linear the reference builds at sparse.py:28-32,
  * here for the int8 MLP linears lin1 (GELU) and lin2 (residual) (modeling/common.py:26).
- * y and residual rows must be 16-byte aligned (ldy, ld_res multiples of 8).
+ * y and residual rows must be 16-byte aligned (ldy, ld_res multiples of 8).  `layout` is the
+ * layout of xq (the weight has its own packed form).
  */
 int samfast_gemm_i8_sparse24_fused(
     const int8_t* xq, const float* sx, const int8_t* wc, const int32_t* widx,
     const float* sw, const float* bias, void* y, int64_t ldy,
     int64_t M, int N, int K, int dtype, int epilogue,
-    const void* residual, int64_t ld_res, void* stream);
+    const void* residual, int64_t ld_res, int layout, void* stream);
 
 #ifdef __cplusplus
 }

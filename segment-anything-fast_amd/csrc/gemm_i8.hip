@@ -55,6 +55,8 @@ struct GemmArgs {
   int64_t ldo;
   int M, N, K;
   int tiles_m, tiles_n;
+  int row_pitch;            // bytes between consecutive rows of X / W: K (row-major) or 64 (K-block major)
+  int64_t x_kstep, w_kstep; // bytes between consecutive 64-byte k tiles: 64, or rows * 64
   const unsigned short* residual;  // EPI_RESIDUAL: (rows, N) bf16, row stride ld_res
   int64_t ld_res;
   const int32_t* dst_row;          // EPI_RESIDUAL: output row per GEMM row, -1 = drop; may be null
@@ -302,7 +304,7 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
     const int row = c >> 2, kc = c & 3;
     if (i < TM) {
       const int gm = min(m0 + row, a.M - 1);
-      ox[i] = gm * a.K + kc * 16;
+      ox[i] = gm * a.row_pitch + kc * 16;
       lx[i] = row * GLD + ((kc ^ lds_swizzle(row)) * 16);
     }
     // W: consecutive chunk groups go to consecutive LDS slots (no write bank conflicts);
@@ -310,7 +312,7 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
     const int slot = row & 127;
     const int wrow = (row & 128) + (slot & 31) * 4 + (slot >> 5);
     const int gn = min(n0 + wrow, a.N - 1);
-    ow[i] = gn * a.K + kc * 16;
+    ow[i] = gn * a.row_pitch + kc * 16;
     lw[i] = GBM * GLD + row * GLD + ((kc ^ lds_swizzle(row)) * 16);
   }
 
@@ -333,8 +335,8 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
   //      the global loads of tile kt+3 - all while the MFMAs of k-step 1 run.
   i32x4 stg_x[TM], stg_w[4];
   auto global_fetch = [&](int kt) {
-    const int8_t* xb = a.x + kt * GBK;  // uniform
-    const int8_t* wb = a.w + kt * GBK;
+    const int8_t* xb = a.x + kt * a.x_kstep;  // uniform
+    const int8_t* wb = a.w + kt * a.w_kstep;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (i < TM) stg_x[i] = *reinterpret_cast<const i32x4*>(xb + ox[i]);
@@ -419,18 +421,18 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
       const int rho = 16 * (wave_u + 4 * i) + (lane >> 2);  // LDS row of this lane's chunk
       const int chunk = (lane & 3) ^ lds_swizzle(rho);
       if (i < GBM / 64) {  // X rows
-        dma_off[i] = min(m0 + rho, a.M - 1) * a.K + chunk * 16;
+        dma_off[i] = min(m0 + rho, a.M - 1) * a.row_pitch + chunk * 16;
       } else {             // W slots (slot s of a 128-column half holds W row (s%32)*4 + s/32)
         const int sl = rho - GBM;
         const int wrow = (sl & 128) + (sl & 31) * 4 + ((sl & 127) >> 5);
-        dma_off[i] = min(n0 + wrow, a.N - 1) * a.K + chunk * 16;
+        dma_off[i] = min(n0 + wrow, a.N - 1) * a.row_pitch + chunk * 16;
       }
     }
     typedef __attribute__((address_space(1))) const void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
     auto dma_issue = [&](int kt, int stage_off) {
-      const int8_t* xb = a.x + kt * GBK;
-      const int8_t* wb = a.w + kt * GBK;
+      const int8_t* xb = a.x + kt * a.x_kstep;
+      const int8_t* wb = a.w + kt * a.w_kstep;
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
         const int8_t* src = (i < GBM / 64 ? xb : wb) + dma_off[i];
@@ -548,8 +550,10 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
 static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t* wq,
                        const float* sw, const float* bias, void* out, int64_t ldo, int64_t M,
                        int N, int K, hipStream_t stream, const void* residual = nullptr,
-                       int64_t ld_res = 0, const int32_t* dst_row = nullptr) {
+                       int64_t ld_res = 0, const int32_t* dst_row = nullptr,
+                       int layout = SAMFAST_LAYOUT_ROWMAJOR) {
   SF_REQUIRE(xq && wq && out, "gemm_i8: null pointer");
+  SF_REQUIRE(layout == SAMFAST_LAYOUT_ROWMAJOR || layout == SAMFAST_LAYOUT_KB64, "gemm_i8: unknown layout %d", layout);
   SF_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_i8: bad shape M=%lld N=%d K=%d", (long long)M, N, K);
   SF_REQUIRE(M < (1ll << 31) - 256, "gemm_i8: M=%lld too large", (long long)M);
   SF_REQUIRE(M * K < (1ll << 31) && (int64_t)N * K < (1ll << 31),
@@ -570,6 +574,11 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   GemmArgs a;
   a.x = xq; a.w = wq; a.out = out; a.sx = sx; a.sw = sw; a.bias = bias;
   a.ldo = ldo; a.M = (int)M; a.N = N; a.K = K;
+  if (layout == SAMFAST_LAYOUT_KB64) {
+    a.row_pitch = GBK; a.x_kstep = M * GBK; a.w_kstep = (int64_t)N * GBK;
+  } else {
+    a.row_pitch = K; a.x_kstep = GBK; a.w_kstep = GBK;
+  }
   a.residual = reinterpret_cast<const unsigned short*>(residual);
   a.ld_res = ld_res; a.dst_row = dst_row;
   if (epi == EPI_RESIDUAL_BF16) {
@@ -629,7 +638,7 @@ extern "C" int samfast_gemm_i8_fused(const int8_t* xq, const float* sx, const in
                                      const float* sw, const float* bias, void* y, int64_t ldy,
                                      int64_t M, int N, int K, int dtype, int epilogue,
                                      const void* residual, int64_t ld_res, const int32_t* dst_row,
-                                     void* stream) {
+                                     int layout, void* stream) {
   using namespace samfast;
   if (dtype != SAMFAST_BF16) {
     set_error("gemm_i8_fused: only bf16 output");
@@ -645,5 +654,5 @@ extern "C" int samfast_gemm_i8_fused(const int8_t* xq, const float* sx, const in
       return SAMFAST_E_INVALID;
   }
   return gemm_common(epi, xq, sx, wq, sw, bias, y, ldy, M, N, K,
-                     reinterpret_cast<hipStream_t>(stream), residual, ld_res, dst_row);
+                     reinterpret_cast<hipStream_t>(stream), residual, ld_res, dst_row, layout);
 }

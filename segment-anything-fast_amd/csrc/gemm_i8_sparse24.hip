@@ -62,6 +62,8 @@ struct SparseArgs {
   int64_t ldo;
   int M, N, K;
   int tiles_x, tiles_w;
+  int x_row_pitch;   // bytes between consecutive X rows: K (row-major) or 64 (K-block major)
+  int64_t x_kstep;   // bytes between consecutive 64-byte k tiles of X: 64, or M * 64
   const unsigned short* residual;
   int64_t ld_res;
 };
@@ -190,7 +192,7 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_kernel(SparseArgs a) {
   for (int i = 0; i < 2; ++i) {
     const int blk = wave_u + 4 * i;  // 1 KB block of the X / Wc tile, 256 B block of the index tile
     const int xr = 16 * blk + (lane >> 2);
-    off_x[i] = min(x0 + xr, a.M - 1) * a.K + (((lane & 3) ^ sp_swizzle_x(xr)) * 16);
+    off_x[i] = min(x0 + xr, a.M - 1) * a.x_row_pitch + (((lane & 3) ^ sp_swizzle_x(xr)) * 16);
     const int slot = 32 * blk + (lane >> 1);
     const int gn = min(w0 + sp_slot_to_row(slot), a.N - 1);
     off_w[i] = gn * 32 + (((lane & 1) ^ sp_swizzle_w(slot)) * 16);
@@ -199,7 +201,7 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_kernel(SparseArgs a) {
   typedef __attribute__((address_space(1))) const void* gptr_t;
   typedef __attribute__((address_space(3))) void* lptr_t;
   auto dma_issue = [&](int kt, int stage_off) {
-    const int8_t* xb = a.x + kt * SBK;
+    const int8_t* xb = a.x + kt * a.x_kstep;
     const int8_t* wb_ = a.wc + (int64_t)kt * a.N * 32;
     const int8_t* ib = reinterpret_cast<const int8_t*>(a.widx) + (int64_t)kt * a.N * 8;
 #pragma unroll
@@ -378,8 +380,11 @@ __global__ __launch_bounds__(256) void prune24_pack_kernel(const int8_t* __restr
 static int sparse_common(int epi, const int8_t* xq, const float* sx, const int8_t* wc,
                          const int32_t* widx, const float* sw, const float* bias, void* out,
                          int64_t ldo, int64_t M, int N, int K, hipStream_t stream,
-                         const void* residual = nullptr, int64_t ld_res = 0) {
+                         const void* residual = nullptr, int64_t ld_res = 0,
+                         int layout = SAMFAST_LAYOUT_ROWMAJOR) {
   SF_REQUIRE(xq && wc && widx && out, "gemm_i8_sparse24: null pointer");
+  SF_REQUIRE(layout == SAMFAST_LAYOUT_ROWMAJOR || layout == SAMFAST_LAYOUT_KB64,
+             "gemm_i8_sparse24: unknown layout %d", layout);
   SF_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_i8_sparse24: bad shape M=%lld N=%d K=%d", (long long)M, N, K);
   SF_REQUIRE(M < (1ll << 31) - 256, "gemm_i8_sparse24: M=%lld too large", (long long)M);
   SF_REQUIRE(M * K < (1ll << 31) && (int64_t)N * 32 < (1ll << 31),
@@ -403,6 +408,8 @@ static int sparse_common(int epi, const int8_t* xq, const float* sx, const int8_
   SparseArgs a;
   a.x = xq; a.wc = wc; a.widx = widx; a.out = out; a.sx = sx; a.sw = sw; a.bias = bias;
   a.ldo = ldo; a.M = (int)M; a.N = N; a.K = K;
+  a.x_row_pitch = layout == SAMFAST_LAYOUT_KB64 ? SBK : K;
+  a.x_kstep = layout == SAMFAST_LAYOUT_KB64 ? M * SBK : SBK;
   a.residual = reinterpret_cast<const unsigned short*>(residual);
   a.ld_res = ld_res;
   a.tiles_x = (int)((M + SBX - 1) / SBX);
@@ -448,7 +455,7 @@ extern "C" int samfast_gemm_i8_sparse24_fused(const int8_t* xq, const float* sx,
                                               const int32_t* widx, const float* sw, const float* bias,
                                               void* y, int64_t ldy, int64_t M, int N, int K, int dtype,
                                               int epilogue, const void* residual, int64_t ld_res,
-                                              void* stream) {
+                                              int layout, void* stream) {
   using namespace samfast;
   if (dtype != SAMFAST_BF16) {
     set_error("gemm_i8_sparse24_fused: only bf16 output");
@@ -464,5 +471,5 @@ extern "C" int samfast_gemm_i8_sparse24_fused(const int8_t* xq, const float* sx,
       return SAMFAST_E_INVALID;
   }
   return sparse_common(epi, xq, sx, wc, widx, sw, bias, y, ldy, M, N, K,
-                       reinterpret_cast<hipStream_t>(stream), residual, ld_res);
+                       reinterpret_cast<hipStream_t>(stream), residual, ld_res, layout);
 }

@@ -32,6 +32,7 @@ struct QuantArgs {
   int64_t M;
   int K;
   float eps;
+  int kb64;  // 1: write xq K-block major, (K/64, M, 64)
 };
 
 SF_DEVICE float wave_sum(float v) {
@@ -75,7 +76,12 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
   const int64_t row = (int64_t)blockIdx.x * kQuantWavesPerBlock + (threadIdx.x >> 6);
   if (row >= a.M) return;  // whole wavefront leaves together
   const int nchunk = a.K >> 3;
-  u32x2* dst = reinterpret_cast<u32x2*>(a.xq + row * (int64_t)a.K);
+  // 8-byte chunk c of the row: row-major at row*K + 8c; K-block major at ((c/8)*M + row)*64 + (c%8)*8
+  auto dst_of = [&](int c) {
+    const int64_t off = a.kb64 ? ((int64_t)(c >> 3) * a.M + row) * 64 + (c & 7) * 8
+                               : row * (int64_t)a.K + (int64_t)c * 8;
+    return reinterpret_cast<u32x2*>(a.xq + off);
+  };
 
   int64_t srow = row;
   if (LN && a.src_row) {
@@ -85,7 +91,7 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
 #pragma unroll
       for (int i = 0; i < NCH; ++i) {
         const int c = lane + i * 64;
-        if (c < nchunk) dst[c] = z;
+        if (c < nchunk) *dst_of(c) = z;
       }
       if (lane == 0) a.sx[row] = 1e-5f / 127.0f;
       return;
@@ -163,7 +169,7 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
         v[2 * j] = bf16_lo_to_f32(buf[i][j]);
         v[2 * j + 1] = bf16_hi_to_f32(buf[i][j]);
       }
-      dst[c] = quantize8(v, scale, inv_scale);
+      *dst_of(c) = quantize8(v, scale, inv_scale);
     }
   }
 }
@@ -190,7 +196,9 @@ static int dispatch_quant(const QuantArgs& a, hipStream_t s) {
 }
 
 static int check_common(const char* who, const void* x, int64_t ldx, const int8_t* xq, const float* sx,
-                        int64_t M, int K, int dtype) {
+                        int64_t M, int K, int dtype, int layout) {
+  SF_REQUIRE(layout == SAMFAST_LAYOUT_ROWMAJOR || (layout == SAMFAST_LAYOUT_KB64 && K % 64 == 0),
+             "%s: layout must be row-major, or K-block major with K %% 64 == 0", who);
   SF_REQUIRE(x && xq && sx, "%s: null pointer", who);
   SF_REQUIRE(M >= 0 && K > 0, "%s: bad shape M=%lld K=%d", who, (long long)M, K);
   if (dtype != SAMFAST_BF16) SF_FAIL(SAMFAST_E_UNSUPPORTED, "%s: only bf16 input", who);
@@ -206,23 +214,24 @@ static int check_common(const char* who, const void* x, int64_t ldx, const int8_
 }  // namespace samfast
 
 extern "C" int samfast_quant_rowwise_i8(const void* x, int64_t ldx, int8_t* xq, float* sx,
-                                        int64_t M, int K, int dtype, void* stream) {
+                                        int64_t M, int K, int dtype, int layout, void* stream) {
   using namespace samfast;
-  const int rc = check_common("quant_rowwise", x, ldx, xq, sx, M, K, dtype);
+  const int rc = check_common("quant_rowwise", x, ldx, xq, sx, M, K, dtype, layout);
   if (rc != SAMFAST_OK) return rc;
   if (M == 0) return SAMFAST_OK;
   QuantArgs a = {};
   a.x = reinterpret_cast<const unsigned short*>(x);
   a.ldx = ldx; a.xq = xq; a.sx = sx; a.M = M; a.K = K;
+  a.kb64 = layout == SAMFAST_LAYOUT_KB64;
   return dispatch_quant<false>(a, reinterpret_cast<hipStream_t>(stream));
 }
 
 extern "C" int samfast_layernorm_quant_i8(const void* x, int64_t ldx, const void* gamma,
                                           const void* beta, float eps, const int32_t* src_row,
                                           int8_t* xq, float* sx, int64_t M, int K, int dtype,
-                                          void* stream) {
+                                          int layout, void* stream) {
   using namespace samfast;
-  const int rc = check_common("layernorm_quant", x, ldx, xq, sx, M, K, dtype);
+  const int rc = check_common("layernorm_quant", x, ldx, xq, sx, M, K, dtype, layout);
   if (rc != SAMFAST_OK) return rc;
   SF_REQUIRE(gamma && beta && aligned16(gamma) && aligned16(beta),
              "layernorm_quant: gamma / beta must be non-null and 16-byte aligned");
@@ -234,5 +243,6 @@ extern "C" int samfast_layernorm_quant_i8(const void* x, int64_t ldx, const void
   a.gamma = reinterpret_cast<const unsigned short*>(gamma);
   a.beta = reinterpret_cast<const unsigned short*>(beta);
   a.src_row = src_row; a.eps = eps;
+  a.kb64 = layout == SAMFAST_LAYOUT_KB64;
   return dispatch_quant<true>(a, reinterpret_cast<hipStream_t>(stream));
 }

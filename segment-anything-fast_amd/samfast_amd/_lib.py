@@ -25,23 +25,24 @@ _SIGNATURES = {
         _i32, [_ptr] * 6 + [_i32] * 5 + [_i64] * 12 + [_i32, _f32, _ptr]),
     "samfast_attn_relpos_bias_fwd": (
         _i32, [_ptr] * 6 + [_i32] * 5 + [_i64] * 18 + [_i32, _f32, _ptr]),
-    "samfast_quant_rowwise_i8": (_i32, [_ptr, _i64, _ptr, _ptr, _i64, _i32, _i32, _ptr]),
+    "samfast_quant_rowwise_i8": (_i32, [_ptr, _i64, _ptr, _ptr, _i64, _i32, _i32, _i32, _ptr]),
     "samfast_gemm_i8_i32": (_i32, [_ptr, _ptr, _ptr, _i64, _i32, _i32, _ptr]),
     "samfast_gemm_i8_scale_bias": (
         _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _ptr]),
     "samfast_layernorm_quant_i8": (
-        _i32, [_ptr, _i64, _ptr, _ptr, _f32, _ptr, _ptr, _ptr, _i64, _i32, _i32, _ptr]),
+        _i32, [_ptr, _i64, _ptr, _ptr, _f32, _ptr, _ptr, _ptr, _i64, _i32, _i32, _i32, _ptr]),
     "samfast_gemm_i8_fused": (
         _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _i32,
-               _ptr, _i64, _ptr, _ptr]),
+               _ptr, _i64, _ptr, _i32, _ptr]),
     "samfast_prune24_pack_i8": (_i32, [_ptr, _ptr, _ptr, _i32, _i32, _ptr]),
     "samfast_gemm_i8_sparse24_i32": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _i32, _i32, _ptr]),
     "samfast_gemm_i8_sparse24_fused": (
         _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _i32,
-               _ptr, _i64, _ptr]),
+               _ptr, _i64, _i32, _ptr]),
 }
 
 EPILOGUE_NONE, EPILOGUE_GELU, EPILOGUE_RESIDUAL = 0, 1, 2
+LAYOUT_ROWMAJOR, LAYOUT_KB64 = 0, 1
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

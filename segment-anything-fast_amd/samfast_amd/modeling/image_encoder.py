@@ -33,6 +33,7 @@ from .. import _lib, flash_4, ops
 from ..flash_4 import _attention_rel_h_rel_w
 from .common import LayerNorm2d, MLPBlock
 
+KB64_OPERANDS = os.environ.get("SAMFAST_KB64", "1") != "0"
 FUSED_BLOCK = bool(int(os.environ.get("SAMFAST_FUSED_BLOCK", 1)))
 
 
@@ -146,6 +147,8 @@ class Block(nn.Module):
         nH = attn.num_heads
         hd = C // nH
         tokens = x.contiguous().view(B * H * W, C)
+        # int8 activations travel K-block major between the quantisers and the GEMMs
+        L = _lib.LAYOUT_KB64 if (C % 64 == 0 and KB64_OPERANDS) else _lib.LAYOUT_ROWMAJOR
         if self.window_size > 0:
             ws = self.window_size
             row_map, _ = ops.window_row_maps(B, H, W, ws, x.device)
@@ -155,20 +158,20 @@ class Block(nn.Module):
             gh, gw = H, W
         N = gh * gw
         # norm1 (+ window partition with zero padding) + qkv's activation quantiser
-        xq, sx = ops.layernorm_quant(tokens, self.norm1.weight, self.norm1.bias, self.norm1.eps, row_map)
-        Bw = xq.shape[0] // N
-        qkv = attn.qkv.linear_fused(xq, sx, _lib.EPILOGUE_NONE)
+        xq, sx = ops.layernorm_quant(tokens, self.norm1.weight, self.norm1.bias, self.norm1.eps, row_map, layout=L)
+        Bw = sx.shape[0] // N
+        qkv = attn.qkv.linear_fused(xq, sx, _lib.EPILOGUE_NONE, layout=L)
         qkv = qkv.view(Bw, N, 3, nH, hd)
         q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
         o = ops.attn_relpos(q, k, v, attn.rel_pos_h, attn.rel_pos_w, (gh, gw), attn.scale)
-        oq, so = ops.quant_rowwise(o.permute(0, 2, 1, 3).reshape(Bw * N, C))
+        oq, so = ops.quant_rowwise(o.permute(0, 2, 1, 3).reshape(Bw * N, C), layout=L)
         # proj + window unpartition + `shortcut + x`
-        tokens = attn.proj.linear_fused(oq, so, _lib.EPILOGUE_RESIDUAL, residual=tokens, dst_row=row_map)
+        tokens = attn.proj.linear_fused(oq, so, _lib.EPILOGUE_RESIDUAL, residual=tokens, dst_row=row_map, layout=L)
         # norm2 + lin1's quantiser, lin1 + GELU, lin2's quantiser, lin2 + `x + mlp(...)`
-        hq, sh = ops.layernorm_quant(tokens, self.norm2.weight, self.norm2.bias, self.norm2.eps)
-        h = mlp.lin1.linear_fused(hq, sh, _lib.EPILOGUE_GELU)
-        gq, sg = ops.quant_rowwise(h)
-        tokens = mlp.lin2.linear_fused(gq, sg, _lib.EPILOGUE_RESIDUAL, residual=tokens, out=tokens)
+        hq, sh = ops.layernorm_quant(tokens, self.norm2.weight, self.norm2.bias, self.norm2.eps, layout=L)
+        h = mlp.lin1.linear_fused(hq, sh, _lib.EPILOGUE_GELU, layout=L)
+        gq, sg = ops.quant_rowwise(h, layout=L)
+        tokens = mlp.lin2.linear_fused(gq, sg, _lib.EPILOGUE_RESIDUAL, residual=tokens, out=tokens, layout=L)
         return tokens.view(B, H, W, C)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:

@@ -155,20 +155,54 @@ def attn_relpos_bias(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     return out
 
 
-def quant_rowwise(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """(M, K) bf16 (row stride free, K contiguous) -> (int8 (M, K), fp32 scales (M,))."""
+def _xq_empty(M: int, K: int, layout: int, device) -> torch.Tensor:
+    """int8 activation buffer: (M, K) row-major, or (K/64, M, 64) K-block major."""
+    if layout == _lib.LAYOUT_KB64:
+        if K % 64 != 0:
+            raise RuntimeError("samfast: the K-block major layout needs K % 64 == 0")
+        return torch.empty((K // 64, M, 64), dtype=torch.int8, device=device)
+    return torch.empty((M, K), dtype=torch.int8, device=device)
+
+
+def to_kb64(q: torch.Tensor) -> torch.Tensor:
+    """(R, K) int8 row-major -> (K/64, R, 64) K-block major copy (weights, once)."""
+    R, K = q.shape
+    return q.view(R, K // 64, 64).permute(1, 0, 2).contiguous()
+
+
+def from_kb64(q: torch.Tensor) -> torch.Tensor:
+    """(K/64, R, 64) K-block major -> (R, K) row-major copy."""
+    KB, R, _ = q.shape
+    return q.permute(1, 0, 2).reshape(R, KB * 64)
+
+
+def _operand_shape(q: torch.Tensor, layout: int) -> Tuple[int, int]:
+    """(rows, K) of an int8 GEMM operand in either layout."""
+    if q.dtype != torch.int8 or not q.is_contiguous():
+        raise RuntimeError("samfast: int8 GEMM operands must be contiguous int8 tensors")
+    if layout == _lib.LAYOUT_KB64:
+        if q.dim() != 3 or q.shape[2] != 64:
+            raise RuntimeError("samfast: a K-block major operand has shape (K/64, rows, 64)")
+        return q.shape[1], q.shape[0] * 64
+    if q.dim() != 2:
+        raise RuntimeError("samfast: a row-major operand has shape (rows, K)")
+    return q.shape[0], q.shape[1]
+
+
+def quant_rowwise(x: torch.Tensor, layout: int = _lib.LAYOUT_ROWMAJOR) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(M, K) bf16 (row stride free, K contiguous) -> (int8 codes in `layout`, fp32 scales (M,))."""
     _require_gpu(x)
     if x.dim() != 2 or x.stride(1) != 1:
         raise RuntimeError("samfast: quant_rowwise needs a 2-D tensor with contiguous rows")
     M, K = x.shape
-    xq = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    xq = _xq_empty(M, K, layout, x.device)
     sx = torch.empty((M,), dtype=torch.float32, device=x.device)
     lib = _lib.load()
     code = _timed(
         "quant_rowwise", 3.0 * M * K + 4.0 * M, "byte",
         lambda: lib.samfast_quant_rowwise_i8(
             x.data_ptr(), x.stride(0), xq.data_ptr(), sx.data_ptr(), M, K, _dtype_code(x),
-            _stream()))
+            int(layout), _stream()))
     _lib.check(code, "quant_rowwise_i8")
     return xq, sx
 
@@ -218,7 +252,8 @@ def gemm_i8_scale_bias(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw:
 
 
 def layernorm_quant(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, eps: float,
-                    src_row: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                    src_row: Optional[torch.Tensor] = None,
+                    layout: int = _lib.LAYOUT_ROWMAJOR) -> Tuple[torch.Tensor, torch.Tensor]:
     """LayerNorm over the last axis of x (R, K) bf16, optional row gather (src_row int32 (M,),
     -1 = zero row), then the per-row int8 quantiser.  Returns (int8 (M, K), fp32 (M,))."""
     _require_gpu(x, gamma, beta, src_row)
@@ -230,7 +265,7 @@ def layernorm_quant(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, ep
         raise RuntimeError("samfast: gamma / beta must match x in dtype and length K")
     if src_row is not None and (src_row.dtype != torch.int32 or not src_row.is_contiguous()):
         raise RuntimeError("samfast: src_row must be a contiguous int32 tensor")
-    xq = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    xq = _xq_empty(M, K, layout, x.device)
     sx = torch.empty((M,), dtype=torch.float32, device=x.device)
     lib = _lib.load()
     code = _timed(
@@ -238,7 +273,7 @@ def layernorm_quant(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, ep
         lambda: lib.samfast_layernorm_quant_i8(
             x.data_ptr(), x.stride(0), gamma.contiguous().data_ptr(), beta.contiguous().data_ptr(),
             float(eps), src_row.data_ptr() if src_row is not None else None,
-            xq.data_ptr(), sx.data_ptr(), M, K, _dtype_code(x), _stream()))
+            xq.data_ptr(), sx.data_ptr(), M, K, _dtype_code(x), int(layout), _stream()))
     _lib.check(code, "layernorm_quant_i8")
     return xq, sx
 
@@ -246,16 +281,17 @@ def layernorm_quant(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, ep
 def gemm_i8_fused(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor,
                   bias: Optional[torch.Tensor], epilogue: int,
                   residual: Optional[torch.Tensor] = None, dst_row: Optional[torch.Tensor] = None,
-                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """gemm_i8_scale_bias with a fused tail (see include/samfast.h):
+                  out: Optional[torch.Tensor] = None, layout: int = _lib.LAYOUT_ROWMAJOR) -> torch.Tensor:
+    """gemm_i8_scale_bias with a fused tail (see include/samfast.h); `layout` is the layout of
+    both xq and wq:
     _lib.EPILOGUE_GELU, or _lib.EPILOGUE_RESIDUAL with `residual` (rows_out, N) bf16 and an
     optional int32 row scatter `dst_row` (M,), -1 = dropped.  For RESIDUAL the output has the
     shape of `residual` (and may alias it via `out=residual`)."""
     _require_gpu(xq, sx, wq, sw, bias, residual, dst_row)
-    if not (xq.is_contiguous() and wq.is_contiguous()) or xq.shape[1] != wq.shape[1]:
-        raise RuntimeError("samfast: gemm_i8_fused needs contiguous (M, K) and (N, K)")
-    M, K = xq.shape
-    N = wq.shape[0]
+    M, K = _operand_shape(xq, layout)
+    N, Kw = _operand_shape(wq, layout)
+    if K != Kw:
+        raise RuntimeError("samfast: gemm_i8_fused operands disagree on K")
     if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != M or sw.numel() != N:
         raise RuntimeError("samfast: scales must be fp32 of length M and N")
     if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N):
@@ -284,7 +320,7 @@ def gemm_i8_fused(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torc
             M, N, K, _lib.SAMFAST_BF16, int(epilogue),
             residual.data_ptr() if residual is not None else None,
             residual.stride(0) if residual is not None else 0,
-            dst_row.data_ptr() if dst_row is not None else None, _stream()))
+            dst_row.data_ptr() if dst_row is not None else None, int(layout), _stream()))
     _lib.check(code, "gemm_i8_fused")
     return out
 
@@ -307,10 +343,9 @@ def prune24_pack(wq: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return wc, widx
 
 
-def _check_sparse24(xq: torch.Tensor, wc: torch.Tensor, widx: torch.Tensor) -> Tuple[int, int, int]:
-    if xq.dtype != torch.int8 or xq.dim() != 2 or not xq.is_contiguous():
-        raise RuntimeError("samfast: sparse24 GEMM needs a contiguous int8 (M, K) activation")
-    M, K = xq.shape
+def _check_sparse24(xq: torch.Tensor, wc: torch.Tensor, widx: torch.Tensor,
+                    layout: int = _lib.LAYOUT_ROWMAJOR) -> Tuple[int, int, int]:
+    M, K = _operand_shape(xq, layout)
     if (wc.dtype != torch.int8 or widx.dtype != torch.int32 or wc.dim() != 3 or widx.dim() != 3
             or not (wc.is_contiguous() and widx.is_contiguous())
             or wc.shape[0] * 64 != K or wc.shape[2] != 32
@@ -336,12 +371,14 @@ def gemm_i8_sparse24_i32(xq: torch.Tensor, wc: torch.Tensor, widx: torch.Tensor)
 def gemm_i8_sparse24_fused(xq: torch.Tensor, sx: torch.Tensor, wc: torch.Tensor, widx: torch.Tensor,
                            sw: torch.Tensor, bias: Optional[torch.Tensor], epilogue: int,
                            residual: Optional[torch.Tensor] = None,
-                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """gemm_i8_fused (no row scatter) with the weight in the packed 2:4 form.  The work
+                           out: Optional[torch.Tensor] = None,
+                           layout: int = _lib.LAYOUT_ROWMAJOR) -> torch.Tensor:
+    """gemm_i8_fused (no row scatter) with the weight in the packed 2:4 form; `layout` is the
+    layout of xq.  The work
     reported to record_launches is the multiply-adds the sparse matrix cores execute
     (half the dense count)."""
     _require_gpu(xq, sx, wc, widx, sw, bias, residual)
-    M, N, K = _check_sparse24(xq, wc, widx)
+    M, N, K = _check_sparse24(xq, wc, widx, layout)
     if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != M or sw.numel() != N:
         raise RuntimeError("samfast: scales must be fp32 of length M and N")
     if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N):
@@ -364,7 +401,7 @@ def gemm_i8_sparse24_fused(xq: torch.Tensor, sx: torch.Tensor, wc: torch.Tensor,
             bias.data_ptr() if bias is not None else None, out.data_ptr(), out.stride(0),
             M, N, K, _lib.SAMFAST_BF16, int(epilogue),
             residual.data_ptr() if residual is not None else None,
-            residual.stride(0) if residual is not None else 0, _stream()))
+            residual.stride(0) if residual is not None else 0, int(layout), _stream()))
     _lib.check(code, "gemm_i8_sparse24_fused")
     return out
 

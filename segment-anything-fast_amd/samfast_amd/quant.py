@@ -23,7 +23,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
-from ._lib import EPILOGUE_NONE
+from ._lib import EPILOGUE_NONE, LAYOUT_KB64, LAYOUT_ROWMAJOR
 from .tools import replace_with_custom_fn_if_matches_filter
 
 
@@ -72,7 +72,8 @@ class Int8LinearBase(nn.Module):
     def weight(self) -> torch.Tensor:
         return self.wq.to(torch.float32) * self.sw[:, None]
 
-    def linear_fused(self, xq, sx, epilogue, residual=None, dst_row=None, out=None):
+    def linear_fused(self, xq, sx, epilogue, residual=None, dst_row=None, out=None,
+                     layout=LAYOUT_ROWMAJOR):
         raise NotImplementedError
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -92,6 +93,7 @@ class Int8DynamicLinear(Int8LinearBase):
                  bias: Optional[torch.Tensor]) -> None:
         super().__init__(in_features, out_features, sw, bias)
         self.register_buffer("wq", wq)
+        self._wq_kb64 = None  # derived K-block major copy, not part of the state dict
 
     @classmethod
     def from_float(cls, linear: nn.Linear) -> "Int8DynamicLinear":
@@ -100,10 +102,17 @@ class Int8DynamicLinear(Int8LinearBase):
 
     def linear_fused(self, xq: torch.Tensor, sx: torch.Tensor, epilogue: int,
                      residual: Optional[torch.Tensor] = None, dst_row: Optional[torch.Tensor] = None,
-                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """The GEMM + epilogue on already quantised rows (see ops.gemm_i8_fused)."""
-        return ops.gemm_i8_fused(xq, sx, self.wq, self.sw, self.bias_f32, epilogue,
-                                 residual=residual, dst_row=dst_row, out=out)
+                     out: Optional[torch.Tensor] = None, layout: int = LAYOUT_ROWMAJOR) -> torch.Tensor:
+        """The GEMM + epilogue on already quantised rows (see ops.gemm_i8_fused); `layout` is
+        the layout xq comes in.  The K-block major copy of the weight is made on first use."""
+        if layout == LAYOUT_KB64:
+            if self._wq_kb64 is None or self._wq_kb64.device != self.wq.device:
+                self._wq_kb64 = ops.to_kb64(self.wq)
+            w = self._wq_kb64
+        else:
+            w = self.wq
+        return ops.gemm_i8_fused(xq, sx, w, self.sw, self.bias_f32, epilogue,
+                                 residual=residual, dst_row=dst_row, out=out, layout=layout)
 
     def extra_repr(self) -> str:
         return f"in_features={self.in_features}, out_features={self.out_features}, int8 dynamic"

@@ -89,11 +89,12 @@ class Int8Sparse24Linear(Int8LinearBase):
             out.scatter_(2, col, vals[..., e].permute(1, 0, 2, 3).reshape(N, KB, 16))
         return out.reshape(N, KB * 64)
 
-    def linear_fused(self, xq, sx, epilogue, residual=None, dst_row=None, out=None):
+    def linear_fused(self, xq, sx, epilogue, residual=None, dst_row=None, out=None,
+                     layout=_lib.LAYOUT_ROWMAJOR):
         if dst_row is not None:
             raise RuntimeError("samfast: the sparse GEMM has no row scatter")
         return ops.gemm_i8_sparse24_fused(xq, sx, self.wc, self.widx, self.sw, self.bias_f32,
-                                          epilogue, residual=residual, out=out)
+                                          epilogue, residual=residual, out=out, layout=layout)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "

@@ -44,8 +44,12 @@ def test_argument_validation_without_gpu():
     p += (-p) % 16
     rc = lib.samfast_gemm_i8_i32(p, p, p, 16, 16, 100, None)
     assert rc == -1 and b"multiple of 64" in lib.samfast_last_error()
-    rc = lib.samfast_quant_rowwise_i8(p, 12, p, p, 4, 12, 0, None)
+    rc = lib.samfast_quant_rowwise_i8(p, 12, p, p, 4, 12, 0, 0, None)
     assert rc == -1 and b"multiple of 8" in lib.samfast_last_error()
+    rc = lib.samfast_quant_rowwise_i8(p, 96, p, p, 4, 96, 0, 1, None)  # K-block major needs K % 64 == 0
+    assert rc == -1 and b"K-block major" in lib.samfast_last_error()
+    rc = lib.samfast_gemm_i8_fused(p, p, p, p, None, p, 64, 4, 64, 256, 0, 0, None, 0, None, 7, None)
+    assert rc == -1 and b"layout" in lib.samfast_last_error()
     strides = [0] * 12
     rc = lib.samfast_attn_relpos_fwd(p, p, p, p, p, p, 1, 1, 10, 10, 48, *strides, 0, 0.125, None)
     assert rc == -2 and b"head_dim" in lib.samfast_last_error()

@@ -192,3 +192,44 @@ def test_gemm_fused_gelu_and_residual():
     got = ops.gemm_i8_fused(*args, _lib.EPILOGUE_RESIDUAL, residual=buf, dst_row=dst.cuda(), out=buf).cpu()
     ref = (lin_ref[keep].float() + res2.float()).to(torch.bfloat16)
     assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 264, 256), (777, 3840, 1280), (130, 1280, 5120)])
+def test_kblock_major_layout_matches_row_major(M, N, K):
+    """The K-block major operand layout is a pure re-arrangement: quantiser codes equal the
+    row-major ones after permutation, and the fused GEMM gives the same bits in both layouts."""
+    from samfast_amd import _lib, ops
+    from samfast_amd.quant import quantize_weight_per_channel
+    print(f"case kb64 M={M} N={N} K={K}", flush=True)
+    x, w, b = linear_inputs(M, K, N, seed=M + N + 1)
+    xc = x.cuda()
+    xq, sx = ops.quant_rowwise(xc)
+    xq_kb, sx_kb = ops.quant_rowwise(xc, layout=_lib.LAYOUT_KB64)
+    assert xq_kb.shape == (K // 64, M, 64)
+    assert torch.equal(ops.from_kb64(xq_kb), xq) and torch.equal(sx, sx_kb)
+    g = torch.Generator().manual_seed(5)
+    gamma = (1 + 0.1 * torch.randn(K, generator=g)).to(torch.bfloat16).cuda()
+    beta = (0.1 * torch.randn(K, generator=g)).to(torch.bfloat16).cuda()
+    rows = torch.randint(-1, M, (M + 7,), generator=g, dtype=torch.int32).cuda()
+    a_q, a_s = ops.layernorm_quant(xc, gamma, beta, 1e-6, rows)
+    b_q, b_s = ops.layernorm_quant(xc, gamma, beta, 1e-6, rows, layout=_lib.LAYOUT_KB64)
+    assert torch.equal(ops.from_kb64(b_q), a_q) and torch.equal(a_s, b_s)
+
+    wq, sw = quantize_weight_per_channel(w)
+    wq, sw, bias = wq.cuda(), sw.cuda(), b.float().cuda()
+    wq_kb = ops.to_kb64(wq)
+    assert torch.equal(ops.from_kb64(wq_kb), wq)
+    res = torch.randn((M, N), generator=g).to(torch.bfloat16).cuda()
+    for epi, kw in ((_lib.EPILOGUE_NONE, {}), (_lib.EPILOGUE_GELU, {}),
+                    (_lib.EPILOGUE_RESIDUAL, {"residual": res})):
+        y0 = ops.gemm_i8_fused(xq, sx, wq, sw, bias, epi, **kw)
+        y1 = ops.gemm_i8_fused(xq_kb, sx, wq_kb, sw, bias, epi, layout=_lib.LAYOUT_KB64, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(y0.view(torch.int16), y1.view(torch.int16)), epi
+    if K >= 256 and K % 128 == 0:
+        wc, widx = ops.prune24_pack(wq)
+        y0 = ops.gemm_i8_sparse24_fused(xq, sx, wc, widx, sw, bias, _lib.EPILOGUE_NONE)
+        y1 = ops.gemm_i8_sparse24_fused(xq_kb, sx, wc, widx, sw, bias, _lib.EPILOGUE_NONE,
+                                        layout=_lib.LAYOUT_KB64)
+        torch.cuda.synchronize()
+        assert torch.equal(y0.view(torch.int16), y1.view(torch.int16))
