@@ -432,122 +432,176 @@ __global__ __launch_bounds__(256, 2) void attn_window_kernel(AttnArgs a) {
   const int lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 31, lh = lane >> 5;
   const int N = a.N;
-  const int bh = blockIdx.x;
+  // all heads of a window run on one XCD: their 2*HD-byte slices of a token share cache lines
+  const unsigned int total = (unsigned int)(a.B * a.nH);
+  const int bh = (int)xcd_contiguous_id(blockIdx.x, total);
+  if ((unsigned int)bh >= total) return;  // uniform over the workgroup
   const int b = bh / a.nH, h = bh % a.nH;
 
   const unsigned short* kbase = a.k + b * a.k_sb + h * a.k_sh;
   const unsigned short* vbase = a.v + b * a.v_sb + h * a.v_sh;
   const unsigned short* qbase = a.q + b * a.q_sb + h * a.q_sh;
 
-  // ---- K rows -> LDS; V 4x8 blocks -> transposed LDS (zero beyond N) -----------
+  // ---- requests that do not depend on the staged K / V go out first: the query rows of this
+  //      wave's (up to two) tiles and, for the fused form, the table fragments ---------------
+  const int ntq = (N + 31) / 32;
+  const int nsteps = (N + 15) / 16;
+  unsigned short* X = reinterpret_cast<unsigned short*>(lds + C::X_OFF + wave * C::XBYTES_WAVE);
+  bf16x8 qf0[C::KS], qf1[C::KS];
   {
-    const int nch = N * (HD / 8);
-    for (int c = tid; c < nch; c += 256) {
-      const int row = c / (HD / 8), col = c % (HD / 8);
-      const u32x4 w = *reinterpret_cast<const u32x4*>(kbase + (int64_t)row * a.k_sn + col * 8);
-      *reinterpret_cast<u32x4*>(kl + (row * C::KSTR + col * 8) * 2) = w;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int qcu = min(32 * (wave + 4 * u) + lr, N - 1);
+      const unsigned short* qp = qbase + (int64_t)qcu * a.q_sn + 8 * lh;
+#pragma unroll
+      for (int s = 0; s < C::KS; ++s) (u ? qf1 : qf0)[s] = load_bf16x8_global(qp + 16 * s);
     }
+  }
+  bf16x8 tab_h[FUSED ? C::KS : 1], tab_w[FUSED ? C::KS : 1];
+  if (FUSED) {
+    const int rowh = min(lr, 2 * a.gh - 2), roww = min(lr, 2 * a.gw - 2);
+#pragma unroll
+    for (int s = 0; s < C::KS; ++s) {
+      tab_h[s] = load_bf16x8_global(a.rh + rowh * HD + 16 * s + 8 * lh);
+      tab_w[s] = load_bf16x8_global(a.rw + roww * HD + 16 * s + 8 * lh);
+    }
+  }
+  u32x4 bias_h[2], bias_w[2];
+  // ---- K rows -> LDS; V 4x8 blocks -> transposed LDS (zero beyond N).  Every global load
+  //      of the staging is in flight before the first LDS store --------------------------
+  {
+    constexpr int KCH = (C::NMAX * (HD / 8) + 255) / 256;            // 16-byte K chunks per thread
+    constexpr int VBL = (4 * ((C::NMAX + 15) / 16) * (HD / 8) + 255) / 256;  // 4x8 V blocks per thread
+    const int nch = N * (HD / 8);
     const int nkg = 4 * ((N + 15) / 16);  // key groups of 4, up to the 16-key step boundary
     const int nblk = nkg * (HD / 8);
-    for (int blk = tid; blk < nblk; blk += 256) {
-      const int kg = blk % nkg, dg = blk / nkg;
-      u32x4 in[4];
+    u32x4 kreg[KCH];
+    u32x4 vreg[VBL][4];
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = min(tid + 256 * i, nch - 1);
+      const int row = c / (HD / 8), col = c % (HD / 8);
+      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)row * a.k_sn + col * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VBL; ++i) {
+      const int blk = min(tid + 256 * i, nblk - 1);
+      const int kg = blk / (HD / 8), dg = blk % (HD / 8);  // lanes walk along a V row: coalesced
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
         const int key = 4 * kg + kk;
-        u32x4 w = {0u, 0u, 0u, 0u};
-        if (key < N) w = *reinterpret_cast<const u32x4*>(vbase + (int64_t)key * a.v_sn + dg * 8);
-        in[kk] = w;
+        const u32x4 w = *reinterpret_cast<const u32x4*>(vbase + (int64_t)min(key, N - 1) * a.v_sn + dg * 8);
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        vreg[i][kk] = key < N ? w : z;
       }
-      u32x2 t[8];
-      transpose_4x8(in, t);
+    }
+    // ---- bias operands of both tiles, computed while the staging loads are in flight:
+    //      lane (query, lh) element e <-> slot 8*lh + e --------------------------------------
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        *reinterpret_cast<u32x2*>(vl + ((dg * 8 + i) * C::VSTR + 4 * kg) * 2) = t[i];
+    for (int u = 0; u < 2; ++u) {
+      if (wave + 4 * u < ntq) {  // uniform
+        const int qcu = min(32 * (wave + 4 * u) + lr, N - 1);
+        const int qh = qcu / a.gw, qw = qcu - qh * a.gw;
+        unsigned int bhw[4], bww[4];
+        if (FUSED) {
+          // Th[rel][q], Tw[rel][q] for rel in [0,32): one MFMA row tile each, staged one after
+          // the other through the wave's scratch rows
+          f32x16 th, tw;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) { th[r] = 0.f; tw[r] = 0.f; }
+#pragma unroll
+          for (int s = 0; s < C::KS; ++s) {
+            th = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tab_h[s], (u ? qf1 : qf0)[s], th, 0, 0, 0);
+            tw = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tab_w[s], (u ? qf1 : qf0)[s], tw, 0, 0, 0);
+          }
+#pragma unroll
+          for (int which = 0; which < 2; ++which) {
+            const int g = which ? a.gw : a.gh;
+            const int qpos = which ? qw : qh;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int rel = 8 * (r >> 2) + 4 * lh + (r & 3);
+              const float val = (which ? tw[r] : th[r]) * a.inv_scale;
+              X[lr * C::XSTR + rel] = (unsigned short)f32_to_bf16_bits(val);
+            }
+            wave_lds_fence();
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              unsigned int pk2 = 0u;
+#pragma unroll
+              for (int v = 0; v < 2; ++v) {
+                const int slot = 8 * lh + 2 * i + v;
+                // unconditional read at a clamped position, then select
+                const unsigned int raw = X[lr * C::XSTR + max(0, min(qpos - slot + g - 1, 31))];
+                pk2 |= ((slot < g) ? raw : 0u) << (16 * v);
+              }
+              if (which) bww[i] = pk2; else bhw[i] = pk2;
+            }
+            wave_lds_fence();
+          }
+        } else {
+          const unsigned short* rhp = a.rh + b * a.rh_sb + h * a.rh_sh + (int64_t)qcu * a.rh_sn;
+          const unsigned short* rwp = a.rw + b * a.rw_sb + h * a.rw_sh + (int64_t)qcu * a.rw_sn;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float fh[2] = {0.f, 0.f}, fw[2] = {0.f, 0.f};
+#pragma unroll
+            for (int v = 0; v < 2; ++v) {
+              const int slot = 8 * lh + 2 * i + v;
+              const float rh_raw = bf16_bits_to_f32(rhp[min(slot, a.gh - 1)]) * a.inv_scale;
+              const float rw_raw = bf16_bits_to_f32(rwp[min(slot, a.gw - 1)]) * a.inv_scale;
+              fh[v] = (slot < a.gh) ? rh_raw : 0.f;
+              fw[v] = (slot < a.gw) ? rw_raw : 0.f;
+            }
+            bhw[i] = pack_bf16x2(fh[0], fh[1]);
+            bww[i] = pack_bf16x2(fw[0], fw[1]);
+          }
+        }
+        if (lh == 1) bhw[3] = (bhw[3] & 0xffffu) | 0xF1490000u;  // slot 15 = -1e30 (bf16 0xF149)
+        const u32x4 bhv = {bhw[0], bhw[1], bhw[2], bhw[3]};
+        const u32x4 bwv = {bww[0], bww[1], bww[2], bww[3]};
+        bias_h[u] = bhv;
+        bias_w[u] = bwv;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + 256 * i;
+      if (c < nch) {
+        const int row = c / (HD / 8), col = c % (HD / 8);
+        *reinterpret_cast<u32x4*>(kl + (row * C::KSTR + col * 8) * 2) = kreg[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VBL; ++i) {
+      const int blk = tid + 256 * i;
+      if (blk < nblk) {
+        const int kg = blk / (HD / 8), dg = blk % (HD / 8);  // lanes walk along a V row: coalesced
+        u32x2 t[8];
+        transpose_4x8(vreg[i], t);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          *reinterpret_cast<u32x2*>(vl + ((dg * 8 + j) * C::VSTR + 4 * kg) * 2) = t[j];
+      }
     }
   }
   __syncthreads();
 
-  const int ntq = (N + 31) / 32;
-  const int nsteps = (N + 15) / 16;
-  unsigned short* X = reinterpret_cast<unsigned short*>(lds + C::X_OFF + wave * C::XBYTES_WAVE);
-
-  for (int t = wave; t < ntq; t += 4) {  // wave-uniform
+  for (int t = wave; t < ntq; t += 4) {  // wave-uniform; at most two tiles per wave
+    const int u = (t - wave) >> 2;
     const int qi = 32 * t + lr;
     const bool q_valid = qi < N;
-    const int qc = min(qi, N - 1);
-    const int qh = qc / a.gw, qw = qc - qh * a.gw;
-
     bf16x8 qf[C::KS];
-    {
-      const unsigned short* qp = qbase + (int64_t)qc * a.q_sn + 8 * lh;
+    if (u == 0) {
+#pragma unroll
+      for (int s = 0; s < C::KS; ++s) qf[s] = qf0[s];
+    } else {  // the second tile's rows are fetched again (cache-resident by now) rather than held
+      const unsigned short* qp = qbase + (int64_t)min(qi, N - 1) * a.q_sn + 8 * lh;
 #pragma unroll
       for (int s = 0; s < C::KS; ++s) qf[s] = load_bf16x8_global(qp + 16 * s);
     }
-
-    // ---- bias operands: lane (query, lh) element e <-> slot 8*lh + e -----------
-    unsigned int bhw[4], bww[4];
-    if (FUSED) {
-      // Th[rel][q], Tw[rel][q] for rel in [0,32): one MFMA row tile each, staged
-      // one after the other through the wave's scratch rows
-      f32x16 th, tw;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { th[r] = 0.f; tw[r] = 0.f; }
-      const int rowh = min(lr, 2 * a.gh - 2), roww = min(lr, 2 * a.gw - 2);
-#pragma unroll
-      for (int s = 0; s < C::KS; ++s) {
-        const bf16x8 ah = load_bf16x8_global(a.rh + rowh * HD + 16 * s + 8 * lh);
-        const bf16x8 aw = load_bf16x8_global(a.rw + roww * HD + 16 * s + 8 * lh);
-        th = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, qf[s], th, 0, 0, 0);
-        tw = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aw, qf[s], tw, 0, 0, 0);
-      }
-#pragma unroll
-      for (int which = 0; which < 2; ++which) {
-        const int g = which ? a.gw : a.gh;
-        const int qpos = which ? qw : qh;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int rel = 8 * (r >> 2) + 4 * lh + (r & 3);
-          const float val = (which ? tw[r] : th[r]) * a.inv_scale;
-          X[lr * C::XSTR + rel] = (unsigned short)f32_to_bf16_bits(val);
-        }
-        wave_lds_fence();
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          unsigned int pk2 = 0u;
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            const int slot = 8 * lh + 2 * i + u;
-            // unconditional read at a clamped position, then select
-            const unsigned int raw = X[lr * C::XSTR + max(0, min(qpos - slot + g - 1, 31))];
-            pk2 |= ((slot < g) ? raw : 0u) << (16 * u);
-          }
-          if (which) bww[i] = pk2; else bhw[i] = pk2;
-        }
-        wave_lds_fence();
-      }
-    } else {
-      const unsigned short* rhp = a.rh + b * a.rh_sb + h * a.rh_sh + (int64_t)qc * a.rh_sn;
-      const unsigned short* rwp = a.rw + b * a.rw_sb + h * a.rw_sh + (int64_t)qc * a.rw_sn;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float fh[2] = {0.f, 0.f}, fw[2] = {0.f, 0.f};
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const int slot = 8 * lh + 2 * i + u;
-          const float rh_raw = bf16_bits_to_f32(rhp[min(slot, a.gh - 1)]) * a.inv_scale;
-          const float rw_raw = bf16_bits_to_f32(rwp[min(slot, a.gw - 1)]) * a.inv_scale;
-          fh[u] = (slot < a.gh) ? rh_raw : 0.f;
-          fw[u] = (slot < a.gw) ? rw_raw : 0.f;
-        }
-        bhw[i] = pack_bf16x2(fh[0], fh[1]);
-        bww[i] = pack_bf16x2(fw[0], fw[1]);
-      }
-    }
-    if (lh == 1) bhw[3] = (bhw[3] & 0xffffu) | 0xF1490000u;  // slot 15 = -1e30 (bf16 0xF149)
-    const u32x4 bhv = {bhw[0], bhw[1], bhw[2], bhw[3]};
-    const u32x4 bwv = {bww[0], bww[1], bww[2], bww[3]};
-    const bf16x8 bh_op = as_bf16x8(bhv), bw_op = as_bf16x8(bwv);
+    const bf16x8 bh_op = as_bf16x8(u ? bias_h[1] : bias_h[0]);
+    const bf16x8 bw_op = as_bf16x8(u ? bias_w[1] : bias_w[0]);
 
     // ---- S^T tiles --------------------------------------------------------------
     f32x16 s[C::NT];
@@ -648,7 +702,7 @@ static int launch_hd(const AttnArgs& a, bool global_path, hipStream_t stream) {
     hipLaunchKernelGGL((attn_global_kernel<HD, QT, FUSED>), dim3(grid), dim3(256), 0, stream, a);
     return check_launch("attn_global_kernel");
   }
-  const unsigned int grid = (unsigned int)(a.B * a.nH);
+  const unsigned int grid = (unsigned int)((((int64_t)a.B * a.nH + 7) / 8) * 8);
   hipLaunchKernelGGL((attn_window_kernel<HD, FUSED>), dim3(grid), dim3(256), 0, stream, a);
   return check_launch("attn_window_kernel");
 }
