@@ -85,6 +85,28 @@ int samfast_attn_relpos_fwd(
     int dtype, float sm_scale, void* stream);
 
 /*
+ * Windowed attention on image-ordered tokens: window_partition, the attention of every
+ * window and window_unpartition (modeling/image_encoder.py:169-178, helpers :273-323) in one
+ * launch, without materialising the padded windows.  q, k, v, out are (B, nH, img_h*img_w, hd)
+ * views addressed like samfast_attn_relpos_fwd with n = y*img_w + x; the image is cut into
+ * ceil(img_h/ws) x ceil(img_w/ws) windows of ws x ws tokens; positions outside the image are
+ * the reference's zero-padded tokens: they take part as keys / values with the rows
+ * pad_k / pad_v ((nH, hd) each, same element type - for SAM the bf16-rounded k and v bias of
+ * the qkv Linear, which is what a zero input row produces) and produce no output.
+ * rel_pos_h / rel_pos_w: (2*ws-1, hd).  Supported: hd in {64, 80}, ws <= 14, bf16.
+ */
+int samfast_attn_relpos_windowed_fwd(
+    const void* q, const void* k, const void* v,
+    const void* rel_pos_h, const void* rel_pos_w,
+    const void* pad_k, const void* pad_v, void* out,
+    int B, int nH, int img_h, int img_w, int ws, int hd,
+    int64_t q_sb, int64_t q_sh, int64_t q_sn,
+    int64_t k_sb, int64_t k_sh, int64_t k_sn,
+    int64_t v_sb, int64_t v_sh, int64_t v_sn,
+    int64_t o_sb, int64_t o_sh, int64_t o_sn,
+    int dtype, float sm_scale, void* stream);
+
+/*
  * Same attention with the two bias factors already computed by the caller:
  *   rel_h: (B, nH, N, gh) addressed ptr + b*rh_sb + h*rh_sh + n*rh_sn + j
  *   rel_w: (B, nH, N, gw) addressed ptr + b*rw_sb + h*rw_sh + n*rw_sn + j

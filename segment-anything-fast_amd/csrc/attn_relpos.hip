@@ -51,6 +51,12 @@ struct AttnArgs {
   int B, nH, gh, gw, N;
   float c;          // sm_scale * log2(e)
   float inv_scale;  // 1 / sm_scale
+  // window kernel on image-ordered tokens (ws > 0): B counts images of img_h x img_w tokens,
+  // a workgroup's window (iy, ix) covers tokens (iy*ws + y, ix*ws + x); positions outside the
+  // image are padding tokens whose K / V rows are pad_k / pad_v (nH * hd values each)
+  int img_h, img_w, ws, wins_x, wins_y;
+  const unsigned short* pad_k;
+  const unsigned short* pad_v;
 };
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -94,7 +100,10 @@ struct GlobalCfg {
   static constexpr int KSTR = HD + 8;         // K row stride in LDS (elements)
   static constexpr int VSTR = 64 + 8;         // V^T row stride in LDS (elements)
   static constexpr int KBYTES = 64 * KSTR * 2;
-  static constexpr int VBYTES = HD * VSTR * 2;
+  // when HD is not a multiple of 32 the last output tile has spare rows: one extra V^T row of
+  // ones makes the P V product deliver the softmax denominator for free
+  static constexpr bool ONES_ROW = HD % 32 != 0;
+  static constexpr int VBYTES = (HD + (ONES_ROW ? 1 : 0)) * VSTR * 2;
   static constexpr int STAGE = KBYTES + VBYTES;
   static constexpr int RELH_OFF = 2 * STAGE;
   static constexpr int RELH_BYTES = 64 * BM * 4;
@@ -274,6 +283,10 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
     }
   }
   __syncthreads();  // scratch reads done, relhT complete
+  if (C::ONES_ROW && tid < 2 * C::VSTR) {  // the ones row of both stages (never overwritten)
+    const int buf = tid / C::VSTR, col = tid % C::VSTR;
+    *reinterpret_cast<unsigned short*>(lds + buf * C::STAGE + C::KBYTES + (HD * C::VSTR + col) * 2) = 0x3F80;
+  }
   stage_store(0);
   __syncthreads();
 
@@ -302,14 +315,12 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
-      for (int t = 0; t < QT; ++t) s[t][nt] = b1[t][nt];
-#pragma unroll
       for (int ks = 0; ks < C::KS; ++ks) {
         const bf16x8 av = as_bf16x8(*reinterpret_cast<const u32x4*>(
             kl + ((32 * nt + lr) * C::KSTR + 16 * ks + 8 * lh) * 2));
 #pragma unroll
-        for (int t = 0; t < QT; ++t)
-          s[t][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[t][ks], s[t][nt], 0, 0, 0);
+        for (int t = 0; t < QT; ++t)  // the first step takes rel_w / sm_scale as its accumulator input
+          s[t][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[t][ks], ks == 0 ? b1[t][nt] : s[t][nt], 0, 0, 0);
       }
     }
 
@@ -335,9 +346,9 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
         for (int r = 0; r < 16; ++r) {
           const float p = fast_exp2(fmaf(s[t][nt][r], a.c, neg_mrow));
           s[t][nt][r] = p;
-          lsum += p;
+          if (!C::ONES_ROW) lsum += p;
         }
-      l_i[t] = l_i[t] * alpha + lsum;
+      if (!C::ONES_ROW) l_i[t] = l_i[t] * alpha + lsum;
       if (__any(alpha != 1.0f)) {
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt)
@@ -353,7 +364,7 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
       for (int dt = 0; dt < C::DT; ++dt) {
-        const int drow = min(32 * dt + lr, HD - 1);
+        const int drow = min(32 * dt + lr, C::ONES_ROW ? HD : HD - 1);  // row HD: ones
         const unsigned char* vp = vl + (drow * C::VSTR + 16 * j + 4 * lh) * 2;
         const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
         const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 16);
@@ -372,7 +383,17 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
   // ---- epilogue: O = acc / l, 4 adjacent channels per store --------------------
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
-    const float l = l_i[t] + xor32(l_i[t]);
+    float l;
+    if (C::ONES_ROW) {
+      // output row HD (the ones row) = tile DT-1, row HD % 32, held by the lh = (HD % 32) / 4 % 2 lanes
+      constexpr int orow = HD % 32;
+      constexpr int oreg = 4 * (orow / 8) + orow % 4, olh = (orow / 4) % 2;
+      const float own = oacc[t][C::DT - 1][oreg];
+      const float other = xor32(own);
+      l = (lh == olh) ? own : other;
+    } else {
+      l = l_i[t] + xor32(l_i[t]);
+    }
     const float inv = 1.0f / l;
     unsigned short* op = a.out + b * a.o_sb + h * a.o_sh + (int64_t)(q_wg + q_wave + 32 * t + lr) * a.o_sn;
 #pragma unroll
@@ -433,14 +454,31 @@ __global__ __launch_bounds__(256, 2) void attn_window_kernel(AttnArgs a) {
   const int lr = lane & 31, lh = lane >> 5;
   const int N = a.N;
   // all heads of a window run on one XCD: their 2*HD-byte slices of a token share cache lines
-  const unsigned int total = (unsigned int)(a.B * a.nH);
+  const unsigned int total = (unsigned int)((a.ws > 0 ? a.B * a.wins_x * a.wins_y : a.B) * a.nH);
   const int bh = (int)xcd_contiguous_id(blockIdx.x, total);
   if ((unsigned int)bh >= total) return;  // uniform over the workgroup
-  const int b = bh / a.nH, h = bh % a.nH;
+  const int bwin = bh / a.nH, h = bh % a.nH;
+  // image-ordered mode: bwin = (image, window row, window column)
+  int b = bwin, win_y0 = 0, win_x0 = 0;
+  if (a.ws > 0) {
+    const int per_img = a.wins_x * a.wins_y;
+    b = bwin / per_img;
+    const int wi = bwin - b * per_img;
+    win_y0 = (wi / a.wins_x) * a.ws;
+    win_x0 = (wi % a.wins_x) * a.ws;
+  }
+  // token n of the window -> row index inside the (b, head) slice, or -1 for a padding token
+  auto tok_of = [&](int n) {
+    if (a.ws <= 0) return n;
+    const int y = win_y0 + n / a.gw, x = win_x0 + n % a.gw;
+    return (y < a.img_h && x < a.img_w) ? y * a.img_w + x : -1;
+  };
 
   const unsigned short* kbase = a.k + b * a.k_sb + h * a.k_sh;
   const unsigned short* vbase = a.v + b * a.v_sb + h * a.v_sh;
   const unsigned short* qbase = a.q + b * a.q_sb + h * a.q_sh;
+  const unsigned short* kpad = a.ws > 0 ? a.pad_k + h * HD : kbase;
+  const unsigned short* vpad = a.ws > 0 ? a.pad_v + h * HD : vbase;
 
   // ---- requests that do not depend on the staged K / V go out first: the query rows of this
   //      wave's (up to two) tiles and, for the fused form, the table fragments ---------------
@@ -452,7 +490,7 @@ __global__ __launch_bounds__(256, 2) void attn_window_kernel(AttnArgs a) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int qcu = min(32 * (wave + 4 * u) + lr, N - 1);
-      const unsigned short* qp = qbase + (int64_t)qcu * a.q_sn + 8 * lh;
+      const unsigned short* qp = qbase + (int64_t)max(tok_of(qcu), 0) * a.q_sn + 8 * lh;  // padding queries: any row
 #pragma unroll
       for (int s = 0; s < C::KS; ++s) (u ? qf1 : qf0)[s] = load_bf16x8_global(qp + 16 * s);
     }
@@ -481,7 +519,9 @@ __global__ __launch_bounds__(256, 2) void attn_window_kernel(AttnArgs a) {
     for (int i = 0; i < KCH; ++i) {
       const int c = min(tid + 256 * i, nch - 1);
       const int row = c / (HD / 8), col = c % (HD / 8);
-      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)row * a.k_sn + col * 8);
+      const int tok = tok_of(row);
+      const unsigned short* src = tok >= 0 ? kbase + (int64_t)tok * a.k_sn : kpad;
+      kreg[i] = *reinterpret_cast<const u32x4*>(src + col * 8);
     }
 #pragma unroll
     for (int i = 0; i < VBL; ++i) {
@@ -490,7 +530,9 @@ __global__ __launch_bounds__(256, 2) void attn_window_kernel(AttnArgs a) {
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
         const int key = 4 * kg + kk;
-        const u32x4 w = *reinterpret_cast<const u32x4*>(vbase + (int64_t)min(key, N - 1) * a.v_sn + dg * 8);
+        const int tok = tok_of(min(key, N - 1));
+        const unsigned short* src = tok >= 0 ? vbase + (int64_t)tok * a.v_sn : vpad;
+        const u32x4 w = *reinterpret_cast<const u32x4*>(src + dg * 8);
         const u32x4 z = {0u, 0u, 0u, 0u};
         vreg[i][kk] = key < N ? w : z;
       }
@@ -596,7 +638,7 @@ __global__ __launch_bounds__(256, 2) void attn_window_kernel(AttnArgs a) {
 #pragma unroll
       for (int s = 0; s < C::KS; ++s) qf[s] = qf0[s];
     } else {  // the second tile's rows are fetched again (cache-resident by now) rather than held
-      const unsigned short* qp = qbase + (int64_t)min(qi, N - 1) * a.q_sn + 8 * lh;
+      const unsigned short* qp = qbase + (int64_t)max(tok_of(min(qi, N - 1)), 0) * a.q_sn + 8 * lh;
 #pragma unroll
       for (int s = 0; s < C::KS; ++s) qf[s] = load_bf16x8_global(qp + 16 * s);
     }
@@ -672,8 +714,9 @@ __global__ __launch_bounds__(256, 2) void attn_window_kernel(AttnArgs a) {
     }
     const float l = lsum + xor32(lsum);
     const float inv = 1.0f / l;
-    if (q_valid) {
-      unsigned short* op = a.out + b * a.o_sb + h * a.o_sh + (int64_t)qi * a.o_sn;
+    const int otok = q_valid ? tok_of(qi) : -1;  // padding queries produce no output
+    if (otok >= 0) {
+      unsigned short* op = a.out + b * a.o_sb + h * a.o_sh + (int64_t)otok * a.o_sn;
 #pragma unroll
       for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
@@ -702,7 +745,8 @@ static int launch_hd(const AttnArgs& a, bool global_path, hipStream_t stream) {
     hipLaunchKernelGGL((attn_global_kernel<HD, QT, FUSED>), dim3(grid), dim3(256), 0, stream, a);
     return check_launch("attn_global_kernel");
   }
-  const unsigned int grid = (unsigned int)((((int64_t)a.B * a.nH + 7) / 8) * 8);
+  const int64_t wins = a.ws > 0 ? (int64_t)a.B * a.wins_x * a.wins_y : a.B;
+  const unsigned int grid = (unsigned int)(((wins * a.nH + 7) / 8) * 8);
   hipLaunchKernelGGL((attn_window_kernel<HD, FUSED>), dim3(grid), dim3(256), 0, stream, a);
   return check_launch("attn_window_kernel");
 }
@@ -716,8 +760,16 @@ static int attn_dispatch(bool fused, AttnArgs& a, int hd, int dtype, float sm_sc
   if (hd != 64 && hd != 80)
     SF_FAIL(SAMFAST_E_UNSUPPORTED, "attn_relpos: head_dim %d not in {64, 80}", hd);
   SF_REQUIRE((int64_t)a.B * a.nH < (1ll << 24), "attn_relpos: B*nH too large");
+  if (a.ws > 0) {
+    SF_REQUIRE(fused && a.gh == a.ws && a.gw == a.ws && a.img_h > 0 && a.img_w > 0 && a.pad_k && a.pad_v &&
+                   aligned16(a.pad_k) && aligned16(a.pad_v),
+               "attn_relpos_windowed: bad window geometry or padding rows");
+    a.wins_y = (a.img_h + a.ws - 1) / a.ws;
+    a.wins_x = (a.img_w + a.ws - 1) / a.ws;
+    SF_REQUIRE((int64_t)a.B * a.wins_x * a.wins_y * a.nH < (1ll << 30), "attn_relpos_windowed: too many windows");
+  }
   a.N = a.gh * a.gw;
-  const bool global_path = (a.gw == 64) && (a.N % 128 == 0) && (a.gh <= 64);
+  const bool global_path = a.ws <= 0 && (a.gw == 64) && (a.N % 128 == 0) && (a.gh <= 64);
   const bool window_path = (a.gh <= 15) && (a.gw <= 16) && (a.N <= 208);
   if (!global_path && !window_path)
     SF_FAIL(SAMFAST_E_UNSUPPORTED,
@@ -784,4 +836,26 @@ extern "C" int samfast_attn_relpos_bias_fwd(
   SF_REQUIRE(rh_sb >= 0 && rh_sh >= 0 && rh_sn >= 0 && rw_sb >= 0 && rw_sh >= 0 && rw_sn >= 0,
              "attn_relpos_bias: negative bias stride");
   return samfast::attn_dispatch(false, a, hd, dtype, sm_scale, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int samfast_attn_relpos_windowed_fwd(
+    const void* q, const void* k, const void* v, const void* rel_pos_h, const void* rel_pos_w,
+    const void* pad_k, const void* pad_v, void* out,
+    int B, int nH, int img_h, int img_w, int ws, int hd,
+    int64_t q_sb, int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+    int64_t v_sb, int64_t v_sh, int64_t v_sn, int64_t o_sb, int64_t o_sh, int64_t o_sn,
+    int dtype, float sm_scale, void* stream) {
+  using us = unsigned short;
+  samfast::AttnArgs a = {};
+  if (ws <= 0) {
+    samfast::set_error("attn_relpos_windowed: window size must be positive");
+    return SAMFAST_E_INVALID;
+  }
+  a.q = (const us*)q; a.k = (const us*)k; a.v = (const us*)v;
+  a.rh = (const us*)rel_pos_h; a.rw = (const us*)rel_pos_w; a.out = (us*)out;
+  a.pad_k = (const us*)pad_k; a.pad_v = (const us*)pad_v;
+  a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
+  a.B = B; a.nH = nH; a.gh = ws; a.gw = ws; a.img_h = img_h; a.img_w = img_w; a.ws = ws;
+  return samfast::attn_dispatch(true, a, hd, dtype, sm_scale, reinterpret_cast<hipStream_t>(stream));
 }

@@ -23,6 +23,8 @@ _SIGNATURES = {
     "samfast_last_error": (ctypes.c_char_p, []),
     "samfast_attn_relpos_fwd": (
         _i32, [_ptr] * 6 + [_i32] * 5 + [_i64] * 12 + [_i32, _f32, _ptr]),
+    "samfast_attn_relpos_windowed_fwd": (
+        _i32, [_ptr] * 8 + [_i32] * 6 + [_i64] * 12 + [_i32, _f32, _ptr]),
     "samfast_attn_relpos_bias_fwd": (
         _i32, [_ptr] * 6 + [_i32] * 5 + [_i64] * 18 + [_i32, _f32, _ptr]),
     "samfast_quant_rowwise_i8": (_i32, [_ptr, _i64, _ptr, _ptr, _i64, _i32, _i32, _i32, _ptr]),

@@ -34,6 +34,7 @@ from ..flash_4 import _attention_rel_h_rel_w
 from .common import LayerNorm2d, MLPBlock
 
 KB64_OPERANDS = os.environ.get("SAMFAST_KB64", "1") != "0"
+WINDOWS_IN_PLACE = os.environ.get("SAMFAST_WINDOWS_IN_PLACE", "1") != "0"
 FUSED_BLOCK = bool(int(os.environ.get("SAMFAST_FUSED_BLOCK", 1)))
 
 
@@ -140,6 +141,21 @@ class Block(nn.Module):
         return (attn.rel_pos_h.shape[0] == 2 * gh - 1 and attn.rel_pos_w.shape[0] == 2 * gw - 1
                 and ops.attn_supported(gh * gw, (gh, gw), C // attn.num_heads, x.dtype))
 
+    def _pad_rows(self, nH: int, hd: int, device):
+        """(nH, hd) bf16 k and v rows of a zero-padded token: the qkv bias, rounded as the
+        Linear's epilogue rounds it."""
+        bias = self.attn.qkv.bias_f32
+        key = None if bias is None else (bias.data_ptr(), str(device))
+        if getattr(self, "_pad_key", "unset") != key:
+            C = nH * hd
+            if bias is None:
+                pk = pv = torch.zeros((nH, hd), dtype=torch.bfloat16, device=device)
+            else:
+                pk = bias[C:2 * C].to(torch.bfloat16).view(nH, hd).contiguous()
+                pv = bias[2 * C:3 * C].to(torch.bfloat16).view(nH, hd).contiguous()
+            self._pad_key, self._pad_kv = key, (pk, pv)
+        return self._pad_kv
+
     def _forward_int8_fused(self, x: torch.Tensor) -> torch.Tensor:
         """image_encoder.py:167-183 with every step on the HIP kernels."""
         B, H, W, C = x.shape
@@ -149,24 +165,36 @@ class Block(nn.Module):
         tokens = x.contiguous().view(B * H * W, C)
         # int8 activations travel K-block major between the quantisers and the GEMMs
         L = _lib.LAYOUT_KB64 if (C % 64 == 0 and KB64_OPERANDS) else _lib.LAYOUT_ROWMAJOR
-        if self.window_size > 0:
-            ws = self.window_size
+        ws = self.window_size
+        if ws > 0 and not WINDOWS_IN_PLACE:
+            # windows materialised: the partition is a row gather in the LayerNorm+quant kernel,
+            # the unpartition a row scatter in the proj epilogue
             row_map, _ = ops.window_row_maps(B, H, W, ws, x.device)
-            gh = gw = ws
+            N = ws * ws
+            xq, sx = ops.layernorm_quant(tokens, self.norm1.weight, self.norm1.bias, self.norm1.eps, row_map, layout=L)
+            Bw = sx.shape[0] // N
+            qkv = attn.qkv.linear_fused(xq, sx, _lib.EPILOGUE_NONE, layout=L).view(Bw, N, 3, nH, hd)
+            q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+            o = ops.attn_relpos(q, k, v, attn.rel_pos_h, attn.rel_pos_w, (ws, ws), attn.scale)
+            oq, so = ops.quant_rowwise(o.permute(0, 2, 1, 3).reshape(Bw * N, C), layout=L)
+            tokens = attn.proj.linear_fused(oq, so, _lib.EPILOGUE_RESIDUAL, residual=tokens, dst_row=row_map, layout=L)
         else:
-            row_map = None
-            gh, gw = H, W
-        N = gh * gw
-        # norm1 (+ window partition with zero padding) + qkv's activation quantiser
-        xq, sx = ops.layernorm_quant(tokens, self.norm1.weight, self.norm1.bias, self.norm1.eps, row_map, layout=L)
-        Bw = sx.shape[0] // N
-        qkv = attn.qkv.linear_fused(xq, sx, _lib.EPILOGUE_NONE, layout=L)
-        qkv = qkv.view(Bw, N, 3, nH, hd)
-        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
-        o = ops.attn_relpos(q, k, v, attn.rel_pos_h, attn.rel_pos_w, (gh, gw), attn.scale)
-        oq, so = ops.quant_rowwise(o.permute(0, 2, 1, 3).reshape(Bw * N, C), layout=L)
-        # proj + window unpartition + `shortcut + x`
-        tokens = attn.proj.linear_fused(oq, so, _lib.EPILOGUE_RESIDUAL, residual=tokens, dst_row=row_map, layout=L)
+            # norm1 + qkv's activation quantiser, qkv GEMM on the image-ordered tokens
+            xq, sx = ops.layernorm_quant(tokens, self.norm1.weight, self.norm1.bias, self.norm1.eps, layout=L)
+            qkv = attn.qkv.linear_fused(xq, sx, _lib.EPILOGUE_NONE, layout=L).view(B, H * W, 3, nH, hd)
+            q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+            if ws > 0:
+                # the attention kernel cuts the windows itself; the reference's zero-padded tokens
+                # enter as keys / values with the rows a zero input gives the qkv Linear: its bias
+                pad_k, pad_v = self._pad_rows(nH, hd, x.device)
+                o = ops.attn_relpos_windowed(q, k, v, attn.rel_pos_h, attn.rel_pos_w, pad_k, pad_v,
+                                             (H, W), ws, attn.scale).view(B * H * W, C)
+            else:
+                o = ops.attn_relpos(q, k, v, attn.rel_pos_h, attn.rel_pos_w, (H, W), attn.scale)
+                o = o.permute(0, 2, 1, 3).reshape(B * H * W, C)
+            oq, so = ops.quant_rowwise(o, layout=L)
+            # proj + `shortcut + x`
+            tokens = attn.proj.linear_fused(oq, so, _lib.EPILOGUE_RESIDUAL, residual=tokens, layout=L)
         # norm2 + lin1's quantiser, lin1 + GELU, lin2's quantiser, lin2 + `x + mlp(...)`
         hq, sh = ops.layernorm_quant(tokens, self.norm2.weight, self.norm2.bias, self.norm2.eps, layout=L)
         h = mlp.lin1.linear_fused(hq, sh, _lib.EPILOGUE_GELU, layout=L)

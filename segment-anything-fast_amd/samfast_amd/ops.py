@@ -127,6 +127,40 @@ def attn_relpos(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     return out
 
 
+def attn_relpos_windowed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                         rel_pos_h: torch.Tensor, rel_pos_w: torch.Tensor,
+                         pad_k: torch.Tensor, pad_v: torch.Tensor,
+                         grid_hw: Tuple[int, int], window: int, scale: float) -> torch.Tensor:
+    """Windowed attention on image-ordered tokens (partition + attention + unpartition).
+    q, k, v: (B, nH, H*W, hd) views with contiguous hd; pad_k / pad_v: (nH, hd) rows standing
+    for the zero-padded tokens.  Returns (B, H*W, nH, hd) contiguous."""
+    _require_gpu(q, k, v, rel_pos_h, rel_pos_w, pad_k, pad_v)
+    B, nH, N, hd = q.shape
+    H, W = grid_hw
+    if H * W != N:
+        raise RuntimeError("samfast: grid does not match the token count")
+    if tuple(rel_pos_h.shape) != (2 * window - 1, hd) or tuple(rel_pos_w.shape) != (2 * window - 1, hd):
+        raise RuntimeError("samfast: rel_pos tables must be (2*window-1, head_dim)")
+    for t in (pad_k, pad_v):
+        if tuple(t.shape) != (nH, hd) or not t.is_contiguous() or t.dtype != q.dtype:
+            raise RuntimeError("samfast: pad_k / pad_v must be contiguous (nH, hd) tensors of q's dtype")
+    out = torch.empty((B, N, nH, hd), dtype=q.dtype, device=q.device)
+    o = out.permute(0, 2, 1, 3)
+    lib = _lib.load()
+    nwin = B * (-(-H // window)) * (-(-W // window))
+    nt = window * window
+    code = _timed(
+        "attn_window", 4.0 * nwin * nH * nt * nt * hd, "flop",
+        lambda: lib.samfast_attn_relpos_windowed_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), rel_pos_h.contiguous().data_ptr(),
+            rel_pos_w.contiguous().data_ptr(), pad_k.data_ptr(), pad_v.data_ptr(), out.data_ptr(),
+            B, nH, H, W, window, hd,
+            *_bnhd_strides(q), *_bnhd_strides(k), *_bnhd_strides(v), *_bnhd_strides(o),
+            _dtype_code(q), float(scale), _stream()))
+    _lib.check(code, "attn_relpos_windowed_fwd")
+    return out
+
+
 def attn_relpos_bias(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                      rel_h: torch.Tensor, rel_w: torch.Tensor,
                      sm_scale: Optional[float] = None,

@@ -130,3 +130,51 @@ def test_unsupported_shapes_raise():
     t = torch.zeros((19, 48), dtype=torch.bfloat16, device="cuda")
     with pytest.raises(RuntimeError):
         ops.attn_relpos(q, q, q, t, t, (10, 10))
+
+
+@pytest.mark.parametrize("B,nH,H,W,ws,hd", [(2, 3, 20, 17, 14, 64), (1, 2, 64, 64, 14, 80), (2, 2, 9, 9, 3, 64)])
+def test_windowed_on_image_tokens_equals_partitioned_windows(B, nH, H, W, ws, hd):
+    """samfast_attn_relpos_windowed_fwd = window_partition + per-window attention +
+    window_unpartition: same bits as running the window kernel on explicitly partitioned,
+    padded windows whose padding tokens carry the pad rows; and within the attention
+    tolerance of the fp32 oracle on those windows."""
+    from samfast_amd import ops
+    from oracle import relpos_attention as ora
+    print(f"case windowed B={B} nH={nH} H={H} W={W} ws={ws} hd={hd}", flush=True)
+    g = torch.Generator().manual_seed(B + H + W + hd)
+    C = nH * hd
+    qkv = torch.randn((B, H * W, 3, nH, hd), generator=g).to(torch.bfloat16)
+    rph = (torch.randn((2 * ws - 1, hd), generator=g) * 0.02).to(torch.bfloat16)
+    rpw = (torch.randn((2 * ws - 1, hd), generator=g) * 0.02).to(torch.bfloat16)
+    pad_k = torch.randn((nH, hd), generator=g).to(torch.bfloat16)
+    pad_v = torch.randn((nH, hd), generator=g).to(torch.bfloat16)
+    scale = hd ** -0.5
+    dq = qkv.cuda()
+    q, k, v = (dq[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    out = ops.attn_relpos_windowed(q, k, v, rph.cuda(), rpw.cuda(), pad_k.cuda(), pad_v.cuda(), (H, W), ws, scale)
+    torch.cuda.synchronize()
+    assert out.shape == (B, H * W, nH, hd)
+
+    # explicit partition on the CPU: padded positions get (anything, pad_k, pad_v)
+    def part(t, fill):
+        x = t.reshape(B, H, W, C).float()
+        Hp, Wp = -(-H // ws) * ws, -(-W // ws) * ws
+        full = fill.reshape(1, 1, 1, C).float().expand(B, Hp, Wp, C).clone()
+        full[:, :H, :W] = x
+        wins, _ = ora.window_partition(full, ws)
+        return wins.reshape(-1, ws * ws, nH, hd).permute(0, 2, 1, 3).to(torch.bfloat16)
+    zero = torch.zeros(C)
+    qw, kw, vw = part(qkv[:, :, 0], zero), part(qkv[:, :, 1], pad_k), part(qkv[:, :, 2], pad_v)
+    ow = ops.attn_relpos(qw.cuda().contiguous(), kw.cuda().contiguous(), vw.cuda().contiguous(),
+                         rph.cuda(), rpw.cuda(), (ws, ws), scale)
+    torch.cuda.synchronize()
+    ow = ow.permute(0, 2, 1, 3).reshape(-1, ws, ws, C).float().cpu()
+    Hp, Wp = -(-H // ws) * ws, -(-W // ws) * ws
+    back = ora.window_unpartition(ow, ws, (Hp, Wp), (H, W)).reshape(B, H * W, nH, hd)
+    assert torch.equal(out.float().cpu(), back)
+    # oracle on the same windows (fp32): max-abs <= 2e-2, mean-abs <= 1e-3 on the real tokens
+    ref = ora.attention_from_tables(qw, kw, vw, rph, rpw, (ws, ws))
+    ref = ref.permute(0, 2, 1, 3).reshape(-1, ws, ws, C).float()
+    ref = ora.window_unpartition(ref, ws, (Hp, Wp), (H, W)).reshape(B, H * W, nH, hd)
+    err = (out.float().cpu() - ref).abs()
+    assert err.max() <= 2e-2 and err.mean() <= 1e-3, (err.max(), err.mean())
