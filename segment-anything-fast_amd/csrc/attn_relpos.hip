@@ -32,6 +32,7 @@
 //   n%gw == j]; slot 15 of the rel_h half is the padding mask (B = -1e30, A = 1
 //   for key rows >= N).
 #include "samfast_internal.hpp"
+#include <type_traits>
 
 namespace samfast {
 
@@ -313,9 +314,10 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
     // S^T = K Q^T, accumulator initialised with rel_w / sm_scale
     f32x16 s[QT][2];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int ks = 0; ks < C::KS; ++ks) {
+      // the two key half-tiles are independent accumulator chains: alternate them
 #pragma unroll
-      for (int ks = 0; ks < C::KS; ++ks) {
+      for (int nt = 0; nt < 2; ++nt) {
         const bf16x8 av = as_bf16x8(*reinterpret_cast<const u32x4*>(
             kl + ((32 * nt + lr) * C::KSTR + 16 * ks + 8 * lh) * 2));
 #pragma unroll
