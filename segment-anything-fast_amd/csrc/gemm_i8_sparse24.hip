@@ -162,10 +162,106 @@ SF_DEVICE void sp24_epilogue(const SparseArgs& a, i32x16 (&acc)[4][2], int x0, i
   }
 }
 
+// Staged epilogue (bf16 outputs), same scheme as the dense kernel: scales and bias of the tile
+// were fetched by global->LDS loads at kernel start; phase 1 scales the accumulators and writes
+// a row-major 128 (tokens) x 256 (channels) bf16 tile into the LDS that held the operand
+// stages; phase 2 walks it 8 rows at a time with 16 bytes per lane, so every store and
+// residual load instruction covers two whole 512-byte row segments.
+constexpr int SEP_STRIDE = 544;                     // tile row pitch in bytes
+constexpr int SEP_SCALE_BYTES = 512 + 1024 + 1024;  // sx[128], sw[256], bias[256] as fp32
+
+template <int EPI>
+SF_DEVICE void sp24_epilogue_staged(const SparseArgs& a, i32x16 (&acc)[4][2], unsigned char* lds,
+                                    const unsigned char* sc, int x0, int w0, int wa, int wb,
+                                    int lr, int lh, int tid) {
+  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt 0, lgkmcnt 0
+  __builtin_amdgcn_s_barrier();        // nobody reads operand stages any more
+  __builtin_amdgcn_sched_barrier(0);
+
+  const int chunk = tid & 31, rsub = tid >> 5;
+  const int n = w0 + chunk * 8;
+  const bool col_ok = n < a.N;  // N % 8 == 0
+  auto out_row = [&](int p) {
+    const int m = x0 + 8 * p + rsub;
+    return (m < a.M && col_ok) ? m : -1;
+  };
+  u32x4 res[16];
+  if (EPI == SEPI_RESIDUAL) {  // requested before the conversion work, waited for once
+#pragma unroll
+    for (int p = 0; p < 16; ++p) {
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      res[p] = z;
+      const int dr = out_row(p);
+      if (dr >= 0) res[p] = *reinterpret_cast<const u32x4*>(a.residual + (int64_t)dr * a.ld_res + n);
+    }
+  }
+  {
+    float sxs[2];
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) sxs[tb] = *reinterpret_cast<const float*>(sc + (wb * 64 + tb * 32 + lr) * 4);
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        // 8 consecutive channels: acc[2j][tb][4g + 0..3], acc[2j+1][tb][4g + 0..3]
+        const int nl = wa * 128 + 32 * g + 16 * j + 8 * lh;
+        f32x4 swv[2], bv[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          swv[t] = *reinterpret_cast<const f32x4*>(sc + 512 + (nl + 4 * t) * 4);
+          const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+          bv[t] = a.bias ? *reinterpret_cast<const f32x4*>(sc + 1536 + (nl + 4 * t) * 4) : z;
+        }
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) {
+          u32x4 o;
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            float y[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              // three separately rounded fp32 operations (no fused multiply-add)
+              float v = (float)acc[2 * j + t][tb][4 * g + e] * sxs[tb];
+              v = v * swv[t][e];
+              y[e] = v + bv[t][e];
+            }
+            o[2 * t] = pack_bf16x2(y[0], y[1]);
+            o[2 * t + 1] = pack_bf16x2(y[2], y[3]);
+          }
+          if (EPI == SEPI_GELU) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+              o[c] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[c])), gelu_erf(bf16_hi_to_f32(o[c])));
+          }
+          *reinterpret_cast<u32x4*>(lds + (wb * 64 + tb * 32 + lr) * SEP_STRIDE + nl * 2) = o;
+        }
+      }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);  // LDS writes done, residual values arrived
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+
+  unsigned short* outp = reinterpret_cast<unsigned short*>(a.out);
+#pragma unroll
+  for (int p = 0; p < 16; ++p) {
+    const int dr = out_row(p);
+    u32x4 val = *reinterpret_cast<const u32x4*>(lds + (8 * p + rsub) * SEP_STRIDE + chunk * 16);
+    if (EPI == SEPI_RESIDUAL) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        val[c] = pack_bf16x2(bf16_lo_to_f32(val[c]) + bf16_lo_to_f32(res[p][c]),
+                             bf16_hi_to_f32(val[c]) + bf16_hi_to_f32(res[p][c]));
+    }
+    if (dr >= 0) *reinterpret_cast<u32x4*>(outp + (int64_t)dr * a.ldo + n) = val;
+  }
+}
+
 template <int EPI>
 __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_kernel(SparseArgs a) {
   constexpr int NST = S_NST;
-  __shared__ __attribute__((aligned(16))) unsigned char lds[NST * S_STAGE];
+  constexpr bool STAGED = EPI != SEPI_I32;  // epilogue through LDS
+  static_assert(128 * SEP_STRIDE <= NST * S_STAGE, "output tile must fit in the operand stages");
+  __shared__ __attribute__((aligned(16))) unsigned char lds[NST * S_STAGE + (STAGED ? SEP_SCALE_BYTES : 0)];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -259,6 +355,17 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_kernel(SparseArgs a) {
   auto wait_imm = [](int n) constexpr { return 0x0070 | (n & 15) | ((n >> 4) << 14); };
   static_assert((NST - 1) * NLD <= 63, "vmcnt immediate");
 
+  if constexpr (STAGED) {
+    // row scales, column scales and bias of this tile, 4 bytes per lane, straight into LDS; they
+    // are the oldest loads in flight, so every later vmcnt wait covers them
+    unsigned char* sc = lds + NST * S_STAGE;
+    const int mm = min(x0 + (wave_u & 1) * 64 + lane, a.M - 1);
+    const int nn = min(w0 + wave_u * 64 + lane, a.N - 1);
+    __builtin_amdgcn_global_load_lds((gptr_t)(a.sx + mm), (lptr_t)(sc + (wave_u & 1) * 256), 4, 0, 0);
+    __builtin_amdgcn_global_load_lds((gptr_t)(a.sw + nn), (lptr_t)(sc + 512 + wave_u * 256), 4, 0, 0);
+    __builtin_amdgcn_global_load_lds((gptr_t)((a.bias ? a.bias : a.sw) + nn),
+                                     (lptr_t)(sc + 1536 + wave_u * 256), 4, 0, 0);
+  }
   const int nk = a.K / SBK;  // even and >= NST (checked by the host)
   int st[NST];  // st[j] = LDS offset of the stage holding tile kt + j (uniform, rotated)
 #pragma unroll
@@ -325,7 +432,10 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_kernel(SparseArgs a) {
   iteration(kt + 2, C0{}, C0{}, C1{}, C0{});
   iteration(kt + 3, C1{}, C0{}, C0{}, C0{});
 
-  sp24_epilogue<EPI>(a, acc, x0, w0, wa, wb, lr, lh);
+  if constexpr (STAGED)
+    sp24_epilogue_staged<EPI>(a, acc, lds, lds + NST * S_STAGE, x0, w0, wa, wb, lr, lh, tid);
+  else
+    sp24_epilogue<EPI>(a, acc, x0, w0, wa, wb, lr, lh);
 }
 
 // ---- 2:4 pruning + packing --------------------------------------------------------
