@@ -174,7 +174,6 @@ SF_DEVICE void gemm_epilogue(const GemmArgs& a, i32x16 (&acc)[TM][4], int m0, in
 constexpr int EP_STRIDE = 544;                 // tile row pitch in bytes: rows r and r+4 half a bank cycle apart
 constexpr int EP_SCALE_BYTES = 512 + 1024 + 1024;  // sx[128], sw[256], bias[256] as fp32
 constexpr int EP_ROWMAP_BYTES = 512;                // dst_row[128] (EPI_RESIDUAL)
-constexpr int EP_PAD_BYTES = 256;                   // landing pad of the residual prefetch
 
 template <int EPI>
 SF_DEVICE void gemm_epilogue_staged(const GemmArgs& a, i32x16 (&acc)[2][4], unsigned char* lds,
@@ -275,7 +274,7 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
   constexpr int NST = GENERIC ? 2 : (TM == 4 ? 4 : 3);  // LDS stages
   constexpr bool STAGED = !GENERIC && TM == 2 && EPI != EPI_I32;  // epilogue through LDS
   static_assert(!STAGED || 128 * EP_STRIDE <= NST * GSTAGE, "output tile must fit in the operand stages");
-  __shared__ __attribute__((aligned(16))) unsigned char lds[NST * GSTAGE + (STAGED ? EP_SCALE_BYTES + EP_ROWMAP_BYTES + EP_PAD_BYTES : 0)];
+  __shared__ __attribute__((aligned(16))) unsigned char lds[NST * GSTAGE + (STAGED ? EP_SCALE_BYTES + EP_ROWMAP_BYTES : 0)];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -517,28 +516,11 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
     using Yes = std::integral_constant<int, 1>;
     using No = std::integral_constant<int, 0>;
     for (; kt + NST < nk; ++kt) iteration(kt, Yes{}, Yes{}, std::integral_constant<int, NST - 2>{}, No{});
-    // The residual rows of this tile are touched now (one dword per 128-byte line, landing in
-    // an unused LDS pad), so that the epilogue's residual loads find them in L2.
-    constexpr int NPF = (STAGED && EPI == EPI_RESIDUAL_BF16) ? 2 : 0;
-    if constexpr (NPF > 0) {
-      const unsigned char* sc = lds + NST * GSTAGE;
-#pragma unroll
-      for (int i = 0; i < NPF; ++i) {
-        const int line = (wave_u * NPF + i) * 64 + lane;  // 512 lines: 128 rows x 4
-        const int row = min(line >> 2, a.M - 1 - m0);
-        int dr = m0 + row;
-        if (a.dst_row) dr = max(*reinterpret_cast<const int*>(sc + EP_SCALE_BYTES + row * 4), 0);
-        const int col = min(n0 + (line & 3) * 64, a.N - 8);
-        __builtin_amdgcn_global_load_lds((gptr_t)(a.residual + (int64_t)dr * a.ld_res + col),
-                                         (lptr_t)(lds + NST * GSTAGE + EP_SCALE_BYTES + EP_ROWMAP_BYTES), 4, 0, 0);
-      }
-    }
-    using Extra = std::integral_constant<int, NPF>;
     // the last NST iterations fetch nothing; fewer and fewer tiles remain in flight
-    if constexpr (NST == 4) iteration(kt++, No{}, Yes{}, std::integral_constant<int, 2>{}, Extra{});
-    iteration(kt++, No{}, Yes{}, std::integral_constant<int, 1>{}, Extra{});
-    iteration(kt++, No{}, Yes{}, No{}, Extra{});
-    iteration(kt++, No{}, No{}, No{}, Extra{});
+    if constexpr (NST == 4) iteration(kt++, No{}, Yes{}, std::integral_constant<int, 2>{}, No{});
+    iteration(kt++, No{}, Yes{}, std::integral_constant<int, 1>{}, No{});
+    iteration(kt++, No{}, Yes{}, No{}, No{});
+    iteration(kt++, No{}, No{}, No{}, No{});
   }
 
   if constexpr (STAGED)
