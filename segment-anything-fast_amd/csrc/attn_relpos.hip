@@ -413,22 +413,29 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
 }
 
 // =============================================================================
-// window kernel: gh <= 15, gw <= 16, N = gh*gw <= 208; one workgroup per (b, head)
+// window kernel: gh <= 15, gw <= 16, N = gh*gw <= 208; one workgroup per (window, head)
 // =============================================================================
+// Eight wavefronts: all of them stage K / V, wavefront w then owns query tile w (32 queries;
+// 7 tiles for 196 tokens).  Registers are kept under 128 per lane (online softmax over the
+// key tiles instead of holding all scores) so that two workgroups = four wavefronts per SIMD
+// are resident and fill each other's pipeline gaps.
 template <int HD>
 struct WindowCfg {
   static constexpr int KS = HD / 16;
   static constexpr int DT = (HD + 31) / 32;
   static constexpr int NMAX = 208;
-  static constexpr int NT = 7;                 // score tiles of 32 keys
+  static constexpr int NT = 7;                 // key tiles of 32
+  static constexpr int WAVES = 8;
+  static constexpr int THREADS = 64 * WAVES;
   static constexpr int KSTR = HD + 8;
   static constexpr int VSTR = NMAX + 4;
   static constexpr int KBYTES = NMAX * KSTR * 2;
   static constexpr int VBYTES = HD * VSTR * 2;
   static constexpr int XSTR = 34;              // bf16 elements per scratch row
-  static constexpr int XBYTES_WAVE = 32 * XSTR * 2;      // one bias factor at a time
-  static constexpr int X_OFF = KBYTES + VBYTES;
-  static constexpr int LDS_BYTES = X_OFF + 4 * XBYTES_WAVE;
+  static constexpr int XBYTES_WAVE = 32 * XSTR * 2;  // gather scratch, aliases the K area before K is stored
+  static constexpr int LDS_BYTES = KBYTES + VBYTES;
+  static_assert(WAVES * XBYTES_WAVE <= KBYTES, "gather scratch must fit in the K area");
+  static_assert(NT <= WAVES, "one query tile per wavefront");
 };
 
 // one-hot bf16x8: element e is 1.0 iff slot == 8*lh + e
@@ -445,7 +452,7 @@ SF_DEVICE bf16x8 onehot_bf16x8(int slot, int lh) {
 }
 
 template <int HD, bool FUSED>
-__global__ __launch_bounds__(256, 2) void attn_window_kernel(AttnArgs a) {
+__global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(AttnArgs a) {
   using C = WindowCfg<HD>;
   __shared__ __attribute__((aligned(16))) unsigned char lds[C::LDS_BYTES];
   unsigned char* kl = lds;
@@ -482,255 +489,256 @@ __global__ __launch_bounds__(256, 2) void attn_window_kernel(AttnArgs a) {
   const unsigned short* kpad = a.ws > 0 ? a.pad_k + h * HD : kbase;
   const unsigned short* vpad = a.ws > 0 ? a.pad_v + h * HD : vbase;
 
-  // ---- requests that do not depend on the staged K / V go out first: the query rows of this
-  //      wave's (up to two) tiles and, for the fused form, the table fragments ---------------
   const int ntq = (N + 31) / 32;
   const int nsteps = (N + 15) / 16;
-  unsigned short* X = reinterpret_cast<unsigned short*>(lds + C::X_OFF + wave * C::XBYTES_WAVE);
-  bf16x8 qf0[C::KS], qf1[C::KS];
+  const bool has_tile = wave < ntq;  // uniform per wavefront
+  const int qi = 32 * wave + lr;
+  const int qc = min(qi, N - 1);
+
+  // ---- requests first: this wavefront's query rows, then the K / V staging loads ----------
+  bf16x8 qf[C::KS];
   {
+    const unsigned short* qp = qbase + (int64_t)max(tok_of(qc), 0) * a.q_sn + 8 * lh;  // padding queries: any row
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int qcu = min(32 * (wave + 4 * u) + lr, N - 1);
-      const unsigned short* qp = qbase + (int64_t)max(tok_of(qcu), 0) * a.q_sn + 8 * lh;  // padding queries: any row
+    for (int s = 0; s < C::KS; ++s) qf[s] = load_bf16x8_global(qp + 16 * s);
+  }
+  constexpr int KCH = (C::NMAX * (HD / 8) + C::THREADS - 1) / C::THREADS;            // 16-byte K chunks per thread
+  constexpr int VBL = 1;  // 4x8 V blocks per thread in the pipelined pass (196 keys x 80: 490 blocks)
+  const int nch = N * (HD / 8);
+  const int nkg_real = (N + 3) / 4;     // key groups of 4 that hold real keys
+  const int nkg = 4 * ((N + 15) / 16);  // key groups up to the 16-key step boundary: the rest is zeros
+  const int nblk = nkg_real * (HD / 8);
+  u32x4 kreg[KCH];
+  u32x4 vreg[VBL][4];
 #pragma unroll
-      for (int s = 0; s < C::KS; ++s) (u ? qf1 : qf0)[s] = load_bf16x8_global(qp + 16 * s);
+  for (int i = 0; i < KCH; ++i) {
+    const int c = min(tid + C::THREADS * i, nch - 1);
+    const int row = c / (HD / 8), col = c % (HD / 8);
+    const int tok = tok_of(row);
+    const unsigned short* src = tok >= 0 ? kbase + (int64_t)tok * a.k_sn : kpad;
+    kreg[i] = *reinterpret_cast<const u32x4*>(src + col * 8);
+  }
+#pragma unroll
+  for (int i = 0; i < VBL; ++i) {
+    const int blk = min(tid + C::THREADS * i, nblk - 1);
+    const int kg = blk / (HD / 8), dg = blk % (HD / 8);  // lanes walk along a V row: coalesced
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const int key = 4 * kg + kk;
+      const int tok = tok_of(min(key, N - 1));
+      const unsigned short* src = tok >= 0 ? vbase + (int64_t)tok * a.v_sn : vpad;
+      const u32x4 w = *reinterpret_cast<const u32x4*>(src + dg * 8);
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      vreg[i][kk] = key < N ? w : z;
     }
   }
-  bf16x8 tab_h[FUSED ? C::KS : 1], tab_w[FUSED ? C::KS : 1];
-  if (FUSED) {
-    const int rowh = min(lr, 2 * a.gh - 2), roww = min(lr, 2 * a.gw - 2);
-#pragma unroll
-    for (int s = 0; s < C::KS; ++s) {
-      tab_h[s] = load_bf16x8_global(a.rh + rowh * HD + 16 * s + 8 * lh);
-      tab_w[s] = load_bf16x8_global(a.rw + roww * HD + 16 * s + 8 * lh);
-    }
-  }
-  u32x4 bias_h[2], bias_w[2];
-  // ---- K rows -> LDS; V 4x8 blocks -> transposed LDS (zero beyond N).  Every global load
-  //      of the staging is in flight before the first LDS store --------------------------
+
+  // ---- bias operands while the staging loads are in flight: lane (query, lh) element e <->
+  //      slot 8*lh + e.  The gather scratch lives where K will be stored afterwards ----------
+  u32x4 bias_hv, bias_wv;
   {
-    constexpr int KCH = (C::NMAX * (HD / 8) + 255) / 256;            // 16-byte K chunks per thread
-    constexpr int VBL = (4 * ((C::NMAX + 15) / 16) * (HD / 8) + 255) / 256;  // 4x8 V blocks per thread
-    const int nch = N * (HD / 8);
-    const int nkg = 4 * ((N + 15) / 16);  // key groups of 4, up to the 16-key step boundary
-    const int nblk = nkg * (HD / 8);
-    u32x4 kreg[KCH];
-    u32x4 vreg[VBL][4];
+    const int qh = qc / a.gw, qw = qc - qh * a.gw;
+    unsigned int bhw[4] = {0u, 0u, 0u, 0u}, bww[4] = {0u, 0u, 0u, 0u};
+    if (FUSED) {
+      unsigned short* X = reinterpret_cast<unsigned short*>(lds + wave * C::XBYTES_WAVE);
 #pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      const int c = min(tid + 256 * i, nch - 1);
-      const int row = c / (HD / 8), col = c % (HD / 8);
-      const int tok = tok_of(row);
-      const unsigned short* src = tok >= 0 ? kbase + (int64_t)tok * a.k_sn : kpad;
-      kreg[i] = *reinterpret_cast<const u32x4*>(src + col * 8);
-    }
+      for (int which = 0; which < 2; ++which) {
+        // T[rel][q] = <table[rel], q> for rel in [0, 32): one MFMA row tile, staged through the
+        // wave's scratch rows and read back at rel = qpos - slot + g - 1
+        const int g = which ? a.gw : a.gh;
+        const int qpos = which ? qw : qh;
+        const unsigned short* tab = which ? a.rw : a.rh;
+        const int trow = min(lr, 2 * g - 2);
+        f32x16 tacc;
 #pragma unroll
-    for (int i = 0; i < VBL; ++i) {
-      const int blk = min(tid + 256 * i, nblk - 1);
-      const int kg = blk / (HD / 8), dg = blk % (HD / 8);  // lanes walk along a V row: coalesced
+        for (int r = 0; r < 16; ++r) tacc[r] = 0.f;
+        if (has_tile) {
+          bf16x8 tf[C::KS];
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        const int key = 4 * kg + kk;
-        const int tok = tok_of(min(key, N - 1));
-        const unsigned short* src = tok >= 0 ? vbase + (int64_t)tok * a.v_sn : vpad;
-        const u32x4 w = *reinterpret_cast<const u32x4*>(src + dg * 8);
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        vreg[i][kk] = key < N ? w : z;
-      }
-    }
-    // ---- bias operands of both tiles, computed while the staging loads are in flight:
-    //      lane (query, lh) element e <-> slot 8*lh + e --------------------------------------
+          for (int s = 0; s < C::KS; ++s) tf[s] = load_bf16x8_global(tab + trow * HD + 16 * s + 8 * lh);
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      if (wave + 4 * u < ntq) {  // uniform
-        const int qcu = min(32 * (wave + 4 * u) + lr, N - 1);
-        const int qh = qcu / a.gw, qw = qcu - qh * a.gw;
-        unsigned int bhw[4], bww[4];
-        if (FUSED) {
-          // Th[rel][q], Tw[rel][q] for rel in [0,32): one MFMA row tile each, staged one after
-          // the other through the wave's scratch rows
-          f32x16 th, tw;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) { th[r] = 0.f; tw[r] = 0.f; }
-#pragma unroll
-          for (int s = 0; s < C::KS; ++s) {
-            th = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tab_h[s], (u ? qf1 : qf0)[s], th, 0, 0, 0);
-            tw = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tab_w[s], (u ? qf1 : qf0)[s], tw, 0, 0, 0);
-          }
-#pragma unroll
-          for (int which = 0; which < 2; ++which) {
-            const int g = which ? a.gw : a.gh;
-            const int qpos = which ? qw : qh;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int rel = 8 * (r >> 2) + 4 * lh + (r & 3);
-              const float val = (which ? tw[r] : th[r]) * a.inv_scale;
-              X[lr * C::XSTR + rel] = (unsigned short)f32_to_bf16_bits(val);
-            }
-            wave_lds_fence();
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              unsigned int pk2 = 0u;
-#pragma unroll
-              for (int v = 0; v < 2; ++v) {
-                const int slot = 8 * lh + 2 * i + v;
-                // unconditional read at a clamped position, then select
-                const unsigned int raw = X[lr * C::XSTR + max(0, min(qpos - slot + g - 1, 31))];
-                pk2 |= ((slot < g) ? raw : 0u) << (16 * v);
-              }
-              if (which) bww[i] = pk2; else bhw[i] = pk2;
-            }
-            wave_lds_fence();
-          }
-        } else {
-          const unsigned short* rhp = a.rh + b * a.rh_sb + h * a.rh_sh + (int64_t)qcu * a.rh_sn;
-          const unsigned short* rwp = a.rw + b * a.rw_sb + h * a.rw_sh + (int64_t)qcu * a.rw_sn;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            float fh[2] = {0.f, 0.f}, fw[2] = {0.f, 0.f};
-#pragma unroll
-            for (int v = 0; v < 2; ++v) {
-              const int slot = 8 * lh + 2 * i + v;
-              const float rh_raw = bf16_bits_to_f32(rhp[min(slot, a.gh - 1)]) * a.inv_scale;
-              const float rw_raw = bf16_bits_to_f32(rwp[min(slot, a.gw - 1)]) * a.inv_scale;
-              fh[v] = (slot < a.gh) ? rh_raw : 0.f;
-              fw[v] = (slot < a.gw) ? rw_raw : 0.f;
-            }
-            bhw[i] = pack_bf16x2(fh[0], fh[1]);
-            bww[i] = pack_bf16x2(fw[0], fw[1]);
-          }
+          for (int s = 0; s < C::KS; ++s) tacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf[s], qf[s], tacc, 0, 0, 0);
         }
-        if (lh == 1) bhw[3] = (bhw[3] & 0xffffu) | 0xF1490000u;  // slot 15 = -1e30 (bf16 0xF149)
-        const u32x4 bhv = {bhw[0], bhw[1], bhw[2], bhw[3]};
-        const u32x4 bwv = {bww[0], bww[1], bww[2], bww[3]};
-        bias_h[u] = bhv;
-        bias_w[u] = bwv;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int rel = 8 * (r >> 2) + 4 * lh + (r & 3);
+          X[lr * C::XSTR + rel] = (unsigned short)f32_to_bf16_bits(tacc[r] * a.inv_scale);
+        }
+        wave_lds_fence();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          unsigned int pk2 = 0u;
+#pragma unroll
+          for (int v = 0; v < 2; ++v) {
+            const int slot = 8 * lh + 2 * i + v;
+            // unconditional read at a clamped position, then select
+            const unsigned int raw = X[lr * C::XSTR + max(0, min(qpos - slot + g - 1, 31))];
+            pk2 |= ((slot < g) ? raw : 0u) << (16 * v);
+          }
+          if (which) bww[i] = pk2; else bhw[i] = pk2;
+        }
+        wave_lds_fence();
+      }
+    } else {
+      const unsigned short* rhp = a.rh + b * a.rh_sb + h * a.rh_sh + (int64_t)qc * a.rh_sn;
+      const unsigned short* rwp = a.rw + b * a.rw_sb + h * a.rw_sh + (int64_t)qc * a.rw_sn;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float fh[2] = {0.f, 0.f}, fw[2] = {0.f, 0.f};
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+          const int slot = 8 * lh + 2 * i + v;
+          const float rh_raw = bf16_bits_to_f32(rhp[min(slot, a.gh - 1)]) * a.inv_scale;
+          const float rw_raw = bf16_bits_to_f32(rwp[min(slot, a.gw - 1)]) * a.inv_scale;
+          fh[v] = (slot < a.gh) ? rh_raw : 0.f;
+          fw[v] = (slot < a.gw) ? rw_raw : 0.f;
+        }
+        bhw[i] = pack_bf16x2(fh[0], fh[1]);
+        bww[i] = pack_bf16x2(fw[0], fw[1]);
       }
     }
+    if (lh == 1) bhw[3] = (bhw[3] & 0xffffu) | 0xF1490000u;  // slot 15 = -1e30 (bf16 0xF149)
+    const u32x4 bhv = {bhw[0], bhw[1], bhw[2], bhw[3]};
+    const u32x4 bwv = {bww[0], bww[1], bww[2], bww[3]};
+    bias_hv = bhv;
+    bias_wv = bwv;
+  }
+  __syncthreads();  // every wavefront is done with the scratch: K may overwrite it
+
+  // ---- K rows -> LDS; V 4x8 blocks -> transposed LDS (zero beyond N) ----------------------
 #pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      const int c = tid + 256 * i;
-      if (c < nch) {
-        const int row = c / (HD / 8), col = c % (HD / 8);
-        *reinterpret_cast<u32x4*>(kl + (row * C::KSTR + col * 8) * 2) = kreg[i];
-      }
+  for (int i = 0; i < KCH; ++i) {
+    const int c = tid + C::THREADS * i;
+    if (c < nch) {
+      const int row = c / (HD / 8), col = c % (HD / 8);
+      *reinterpret_cast<u32x4*>(kl + (row * C::KSTR + col * 8) * 2) = kreg[i];
     }
+  }
 #pragma unroll
-    for (int i = 0; i < VBL; ++i) {
-      const int blk = tid + 256 * i;
-      if (blk < nblk) {
-        const int kg = blk / (HD / 8), dg = blk % (HD / 8);  // lanes walk along a V row: coalesced
-        u32x2 t[8];
-        transpose_4x8(vreg[i], t);
+  for (int i = 0; i < VBL; ++i) {
+    const int blk = tid + C::THREADS * i;
+    if (blk < nblk) {
+      const int kg = blk / (HD / 8), dg = blk % (HD / 8);
+      u32x2 t[8];
+      transpose_4x8(vreg[i], t);
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          *reinterpret_cast<u32x2*>(vl + ((dg * 8 + j) * C::VSTR + 4 * kg) * 2) = t[j];
-      }
+      for (int j = 0; j < 8; ++j)
+        *reinterpret_cast<u32x2*>(vl + ((dg * 8 + j) * C::VSTR + 4 * kg) * 2) = t[j];
     }
+  }
+  // blocks beyond one per thread (windows of more than 204 tokens only): plain load-store pass
+  for (int blk = tid + C::THREADS * VBL; blk < nblk; blk += C::THREADS) {
+    const int kg = blk / (HD / 8), dg = blk % (HD / 8);
+    u32x4 in[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const int key = 4 * kg + kk;
+      const int tok = tok_of(min(key, N - 1));
+      const unsigned short* src = tok >= 0 ? vbase + (int64_t)tok * a.v_sn : vpad;
+      const u32x4 w = *reinterpret_cast<const u32x4*>(src + dg * 8);
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      in[kk] = key < N ? w : z;
+    }
+    u32x2 t[8];
+    transpose_4x8(in, t);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      *reinterpret_cast<u32x2*>(vl + ((dg * 8 + j) * C::VSTR + 4 * kg) * 2) = t[j];
+  }
+  // key groups past the last real key, up to the 16-key step boundary: zeros
+  for (int idx = tid; idx < (nkg - nkg_real) * HD; idx += C::THREADS) {
+    const int kg = nkg_real + idx / HD, d = idx % HD;
+    const u32x2 z = {0u, 0u};
+    *reinterpret_cast<u32x2*>(vl + (d * C::VSTR + 4 * kg) * 2) = z;
   }
   __syncthreads();
+  if (!has_tile) return;  // the eighth wavefront only helps with the staging
 
-  for (int t = wave; t < ntq; t += 4) {  // wave-uniform; at most two tiles per wave
-    const int u = (t - wave) >> 2;
-    const int qi = 32 * t + lr;
-    const bool q_valid = qi < N;
-    bf16x8 qf[C::KS];
-    if (u == 0) {
-#pragma unroll
-      for (int s = 0; s < C::KS; ++s) qf[s] = qf0[s];
-    } else {  // the second tile's rows are fetched again (cache-resident by now) rather than held
-      const unsigned short* qp = qbase + (int64_t)max(tok_of(min(qi, N - 1)), 0) * a.q_sn + 8 * lh;
-#pragma unroll
-      for (int s = 0; s < C::KS; ++s) qf[s] = load_bf16x8_global(qp + 16 * s);
-    }
-    const bf16x8 bh_op = as_bf16x8(u ? bias_h[1] : bias_h[0]);
-    const bf16x8 bw_op = as_bf16x8(u ? bias_w[1] : bias_w[0]);
+  const bf16x8 bh_op = as_bf16x8(bias_hv), bw_op = as_bf16x8(bias_wv);
 
-    // ---- S^T tiles --------------------------------------------------------------
-    f32x16 s[C::NT];
-    float mx = -3.0e38f;
+  // ---- online softmax over the key tiles: S^T tile, running max, P, O^T += V^T P^T --------
+  f32x16 oacc[C::DT];
 #pragma unroll
-    for (int nt = 0; nt < C::NT; ++nt) {
-      if (32 * nt < N) {  // uniform
-        const int n = 32 * nt + lr;
-        const int nc = min(n, N - 1);
-        f32x16 acc;
+  for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+  float m_run = -3.0e38f, l_run = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < C::KS; ++ks) {
-          const bf16x8 av = as_bf16x8(
-              *reinterpret_cast<const u32x4*>(kl + (nc * C::KSTR + 16 * ks + 8 * lh) * 2));
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[ks], acc, 0, 0, 0);
+  for (int nt = 0; nt < C::NT; ++nt) {
+    if (32 * nt < N) {  // uniform
+      const int n = 32 * nt + lr;
+      const int nc = min(n, N - 1);
+      f32x16 acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < C::KS; ++ks) {
+        const bf16x8 av = as_bf16x8(
+            *reinterpret_cast<const u32x4*>(kl + (nc * C::KSTR + 16 * ks + 8 * lh) * 2));
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[ks], acc, 0, 0, 0);
+      }
+      const int nh = n / a.gw;
+      const bf16x8 ih = onehot_bf16x8(n < N ? nh : 15, lh);
+      const bf16x8 iw = onehot_bf16x8(n < N ? n - nh * a.gw : 99, lh);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ih, bh_op, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(iw, bw_op, acc, 0, 0, 0);
+
+      float mx = acc[0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, acc[r]);
+      mx = fmaxf(mx, xor32(mx));
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = fast_exp2((m_run - m_new) * a.c);
+      const float neg_m = -m_new * a.c;
+      m_run = m_new;
+      float lsum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = fast_exp2(fmaf(acc[r], a.c, neg_m));
+        acc[r] = p;
+        lsum += p;
+      }
+      l_run = l_run * alpha + lsum;
+      if (__any(alpha != 1.0f)) {
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int j = 2 * nt + half;
+        if (j < nsteps) {  // uniform
+          const bf16x8 pk = cvt_bf16x8(acc, 8 * half);
+#pragma unroll
+          for (int dt = 0; dt < C::DT; ++dt) {
+            const int drow = min(32 * dt + lr, HD - 1);
+            const unsigned char* vp = vl + (drow * C::VSTR + 16 * j + 4 * lh) * 2;
+            const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
+            const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 16);
+            const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(w), pk, oacc[dt], 0, 0, 0);
+          }
         }
-        const int nh = n / a.gw;
-        const bf16x8 ih = onehot_bf16x8(n < N ? nh : 15, lh);
-        const bf16x8 iw = onehot_bf16x8(n < N ? n - nh * a.gw : 99, lh);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ih, bh_op, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(iw, bw_op, acc, 0, 0, 0);
-        s[nt] = acc;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, acc[r]);
-      } else {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[nt][r] = -1.0e30f;
       }
     }
-    mx = fmaxf(mx, xor32(mx));
-    const float neg_m = -mx * a.c;
-
-    // ---- P and O^T = V^T P^T, one score tile (two 16-key steps) at a time -----
-    f32x16 oacc[C::DT];
+  }
+  const float l = l_run + xor32(l_run);
+  const float inv = 1.0f / l;
+  const int otok = qi < N ? tok_of(qi) : -1;  // padding queries produce no output
+  if (otok >= 0) {
+    unsigned short* op = a.out + b * a.o_sb + h * a.o_sh + (int64_t)otok * a.o_sn;
 #pragma unroll
     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
-    float lsum = 0.f;
-#pragma unroll
-    for (int nt = 0; nt < C::NT; ++nt) {
-      if (2 * nt < nsteps) {  // uniform
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float p = fast_exp2(fmaf(s[nt][r], a.c, neg_m));
-          s[nt][r] = p;
-          lsum += p;
-        }
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const int j = 2 * nt + half;
-          if (j < nsteps) {  // uniform
-            const bf16x8 pk = cvt_bf16x8(s[nt], 8 * half);
-#pragma unroll
-            for (int dt = 0; dt < C::DT; ++dt) {
-              const int drow = min(32 * dt + lr, HD - 1);
-              const unsigned char* vp = vl + (drow * C::VSTR + 16 * j + 4 * lh) * 2;
-              const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
-              const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 16);
-              const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
-              oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(w), pk, oacc[dt], 0, 0, 0);
-            }
-          }
+      for (int j = 0; j < 4; ++j) {
+        const int d = 32 * dt + 8 * j + 4 * lh;
+        if (d < HD) {
+          const u32x2 o = {pack_bf16x2(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
+                           pack_bf16x2(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
+          *reinterpret_cast<u32x2*>(op + d) = o;
         }
       }
-    }
-    const float l = lsum + xor32(lsum);
-    const float inv = 1.0f / l;
-    const int otok = q_valid ? tok_of(qi) : -1;  // padding queries produce no output
-    if (otok >= 0) {
-      unsigned short* op = a.out + b * a.o_sb + h * a.o_sh + (int64_t)otok * a.o_sn;
-#pragma unroll
-      for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int d = 32 * dt + 8 * j + 4 * lh;
-          if (d < HD) {
-            const u32x2 o = {pack_bf16x2(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
-                             pack_bf16x2(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
-            *reinterpret_cast<u32x2*>(op + d) = o;
-          }
-        }
-    }
   }
 }
 
@@ -749,7 +757,7 @@ static int launch_hd(const AttnArgs& a, bool global_path, hipStream_t stream) {
   }
   const int64_t wins = a.ws > 0 ? (int64_t)a.B * a.wins_x * a.wins_y : a.B;
   const unsigned int grid = (unsigned int)(((wins * a.nH + 7) / 8) * 8);
-  hipLaunchKernelGGL((attn_window_kernel<HD, FUSED>), dim3(grid), dim3(256), 0, stream, a);
+  hipLaunchKernelGGL((attn_window_kernel<HD, FUSED>), dim3(grid), dim3(WindowCfg<HD>::THREADS), 0, stream, a);
   return check_launch("attn_window_kernel");
 }
 
