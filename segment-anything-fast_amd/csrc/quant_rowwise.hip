@@ -46,27 +46,35 @@ SF_DEVICE float wave_max(float v) {
   return v;
 }
 
-// 8 values -> 8 int8 codes packed in 8 bytes
+// 8 values -> 8 int8 codes packed in 8 bytes.
+// Rounding: adding 1.5 * 2^23 to r (|r| <= 127) leaves rint(r) - half to even - in the low
+// mantissa bits, so the low byte of the sum's bit pattern is the int8 code; subtracting the
+// constant again gives rint(r) as a float for the near-tie test.
 SF_DEVICE u32x2 quantize8(const float (&v)[8], float scale, float inv_scale) {
-  float r[8];
+  constexpr float kMagic = 12582912.0f;  // 1.5 * 2^23
+  float m[8];
   bool near_tie = false;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    r[e] = v[e] * inv_scale;
-    const float frac = r[e] - floorf(r[e]);
-    near_tie |= fabsf(frac - 0.5f) < 1e-4f;
+    const float r = v[e] * inv_scale;
+    m[e] = r + kMagic;
+    const float d = r - (m[e] - kMagic);  // r - rint(r), exact
+    near_tie |= fabsf(d) > 0.5f - 1e-4f;
   }
   if (near_tie) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) r[e] = v[e] / scale;  // IEEE division
+    for (int e = 0; e < 8; ++e) m[e] = v[e] / scale + kMagic;  // IEEE division
   }
-  unsigned int p[2] = {0u, 0u};
+  unsigned int b[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int q = (int)rintf(r[e]);
-    p[e >> 2] |= ((unsigned int)(q & 0xff)) << (8 * (e & 3));
-  }
-  const u32x2 o = {p[0], p[1]};
+  for (int e = 0; e < 8; ++e) b[e] = __builtin_bit_cast(unsigned int, m[e]);
+  // byte 0 of each of four words -> one word (v_perm_b32: selector bytes pick from {hi, lo})
+  auto pack4 = [](unsigned int w0, unsigned int w1, unsigned int w2, unsigned int w3) {
+    const unsigned int lo = __builtin_amdgcn_perm(w1, w0, 0x0c0c0400u);  // [w0.b0, w1.b0, 0, 0]
+    const unsigned int hi = __builtin_amdgcn_perm(w3, w2, 0x04000c0cu);  // [0, 0, w2.b0, w3.b0]
+    return lo | hi;
+  };
+  const u32x2 o = {pack4(b[0], b[1], b[2], b[3]), pack4(b[4], b[5], b[6], b[7])};
   return o;
 }
 
