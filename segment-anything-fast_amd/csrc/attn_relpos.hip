@@ -26,7 +26,9 @@
 //   rel_w[q, kw] = T[qw - kw + 63, q] staged through LDS.
 //
 // window kernel (N <= 208, e.g. 14x14): all keys of one (window, head) fit in
-//   LDS; one pass, no online rescaling.  The bias is added BY THE MFMA: the
+//   LDS; eight wavefronts stage them, each then owns one 32-query tile and walks
+//   the key tiles with an online softmax (under 128 registers per lane, so four
+//   wavefronts per SIMD are resident).  The bias is added BY THE MFMA: the
 //   channel axis is extended by 32 slots, B carries [rel_h[q, 0..15] | rel_w[q,
 //   0..15]] / sm_scale in bf16 and A carries the 0/1 indicators [n/gw == j |
 //   n%gw == j]; slot 15 of the rel_h half is the padding mask (B = -1e30, A = 1
