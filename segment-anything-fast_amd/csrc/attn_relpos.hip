@@ -479,9 +479,13 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     win_x0 = (wi % a.wins_x) * a.ws;
   }
   // token n of the window -> row index inside the (b, head) slice, or -1 for a padding token
+  // n / gw for 0 <= n < 256 and gw <= 16 by multiplication (exact in that range)
+  const int gw_magic = 65536 / a.gw + 1;
+  auto div_gw = [&](int n) { return (n * gw_magic) >> 16; };
   auto tok_of = [&](int n) {
     if (a.ws <= 0) return n;
-    const int y = win_y0 + n / a.gw, x = win_x0 + n % a.gw;
+    const int ny = div_gw(n);
+    const int y = win_y0 + ny, x = win_x0 + n - ny * a.gw;
     return (y < a.img_h && x < a.img_w) ? y * a.img_w + x : -1;
   };
 
@@ -539,7 +543,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
   //      slot 8*lh + e.  The gather scratch lives where K will be stored afterwards ----------
   u32x4 bias_hv, bias_wv;
   {
-    const int qh = qc / a.gw, qw = qc - qh * a.gw;
+    const int qh = div_gw(qc), qw = qc - qh * a.gw;
     unsigned int bhw[4] = {0u, 0u, 0u, 0u}, bww[4] = {0u, 0u, 0u, 0u};
     if (FUSED) {
       unsigned short* X = reinterpret_cast<unsigned short*>(lds + wave * C::XBYTES_WAVE);
@@ -679,7 +683,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
             *reinterpret_cast<const u32x4*>(kl + (nc * C::KSTR + 16 * ks + 8 * lh) * 2));
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[ks], acc, 0, 0, 0);
       }
-      const int nh = n / a.gw;
+      const int nh = div_gw(min(n, 255));
       const bf16x8 ih = onehot_bf16x8(n < N ? nh : 15, lh);
       const bf16x8 iw = onehot_bf16x8(n < N ? n - nh * a.gw : 99, lh);
       acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ih, bh_op, acc, 0, 0, 0);
