@@ -51,6 +51,8 @@ def parse():
     p.add_argument("--sparse-mlp", action="store_true",
                    help="lin1 / lin2 magnitude-pruned 2:4 on the sparse int8 matrix cores (the int8 + 2:4 "
                         "configuration); every other Linear dense int8")
+    p.add_argument("--graph", action="store_true",
+                   help="replay the forward as one HIP graph (launch-bound shapes, e.g. vit_b batch 1)")
     p.add_argument("--calibration-copy", action="store_true",
                    help="also run one 1 GiB device-to-device copy (a known-size reference for "
                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -122,7 +124,13 @@ def main():
 
     with torch.no_grad():
         step = lambda: enc(images)
-        sec = time_steps(step, args.steps, args.warmup)
+        if args.graph:
+            from samfast_amd.graphs import GraphedEncoder
+            graphed = GraphedEncoder(enc, images)
+            timed = lambda: graphed(images)
+        else:
+            timed = step
+        sec = time_steps(timed, args.steps, args.warmup)
         out = step()
         finite = bool(torch.isfinite(out.float()).all())
 
@@ -166,6 +174,7 @@ def main():
                                "1024x1024, rel-pos attention + dynamic int8 linears"
                                + (" (lin1 / lin2 pruned 2:4, sparse int8 MFMA)" if args.sparse_mlp else ""),
                    "batch": args.batch, "image": 1024},
+        "hip_graph": bool(args.graph),
         "output_finite": finite,
         "roofline": roofline,
         "kernels": kernels,

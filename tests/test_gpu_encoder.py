@@ -138,3 +138,52 @@ def test_fused_block_equals_module_composition():
         print(f"fused block ws={ws}: cosine {c:.6f} max-abs {d.max().item():.4f} mean-abs {d.mean().item():.5f}",
               flush=True)
         assert c >= 0.9999 and d.mean().item() <= 2e-3
+
+
+class _Trunk(torch.nn.Module):
+    """Encoder without the neck: patch embedding, position embedding and the blocks."""
+
+    def __init__(self, enc):
+        super().__init__()
+        self.enc = enc
+
+    def forward(self, x):
+        x = self.enc.patch_embed(x)
+        if self.enc.pos_embed is not None:
+            x = x + self.enc.pos_embed
+        for blk in self.enc.blocks:
+            x = blk(x)
+        return x
+
+
+def test_graphed_encoder_replays_equal_eager():
+    """HIP-graph replay of the ViT-B encoder (int8 linears).  The trunk (everything on the HIP
+    kernels) must equal the eager result bit for bit on every replay, with eager work and
+    synchronisations between the replays; the whole encoder is compared by cosine because MIOpen's
+    neck convolutions are not run-to-run deterministic and may use another solver under capture."""
+    from samfast_amd import apply_dynamic_quant
+    from samfast_amd.graphs import GraphedEncoder
+    from samfast_amd.synthetic import make_images
+    enc, _, _ = _vit_b()
+    enc = enc.eval().to(torch.bfloat16).cuda()
+    apply_dynamic_quant(enc)
+    trunk = _Trunk(enc)
+    xs = [make_images(1, seed=s).to(torch.bfloat16).cuda() for s in (1, 2, 3)]
+    with torch.no_grad():
+        eager = [trunk(x).clone() for x in xs]
+        eager_full = [enc(x).clone() for x in xs]
+    g = GraphedEncoder(trunk, xs[0])
+    gf = GraphedEncoder(enc, xs[0])
+    for rep in range(2):
+        for x, ref, ref_full in zip(xs, eager, eager_full):
+            out = g(x).clone()
+            full = gf(x).clone()
+            torch.cuda.synchronize()
+            assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), rep
+            assert _cos(full, ref_full) >= 0.9995  # MIOpen may pick another solver while capturing
+            with torch.no_grad():  # eager work between replays
+                again = trunk(x)
+            torch.cuda.synchronize()
+            assert torch.equal(again.view(torch.int16), ref.view(torch.int16))
+    with pytest.raises(RuntimeError, match="recorded for"):
+        g(torch.zeros((2, 3, 1024, 1024), dtype=torch.bfloat16, device="cuda"))
