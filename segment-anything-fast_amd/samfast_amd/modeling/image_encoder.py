@@ -145,7 +145,7 @@ class Block(nn.Module):
         """(nH, hd) bf16 k and v rows of a zero-padded token: the qkv bias, rounded as the
         Linear's epilogue rounds it."""
         bias = self.attn.qkv.bias_f32
-        key = None if bias is None else (bias.data_ptr(), str(device))
+        key = None if bias is None else (bias.data_ptr(), self.attn.qkv.bias_bits._version, str(device))
         if getattr(self, "_pad_key", "unset") != key:
             C = nH * hd
             if bias is None:

@@ -94,6 +94,7 @@ class Int8DynamicLinear(Int8LinearBase):
         super().__init__(in_features, out_features, sw, bias)
         self.register_buffer("wq", wq)
         self._wq_kb64 = None  # derived K-block major copy, not part of the state dict
+        self._wq_kb64_key = None
 
     @classmethod
     def from_float(cls, linear: nn.Linear) -> "Int8DynamicLinear":
@@ -106,8 +107,9 @@ class Int8DynamicLinear(Int8LinearBase):
         """The GEMM + epilogue on already quantised rows (see ops.gemm_i8_fused); `layout` is
         the layout xq comes in.  The K-block major copy of the weight is made on first use."""
         if layout == LAYOUT_KB64:
-            if self._wq_kb64 is None or self._wq_kb64.device != self.wq.device:
-                self._wq_kb64 = ops.to_kb64(self.wq)
+            key = (self.wq.data_ptr(), self.wq._version, str(self.wq.device))
+            if self._wq_kb64 is None or self._wq_kb64_key != key:  # rebuilt after load_state_dict / .to()
+                self._wq_kb64, self._wq_kb64_key = ops.to_kb64(self.wq), key
             w = self._wq_kb64
         else:
             w = self.wq

@@ -187,3 +187,29 @@ def test_graphed_encoder_replays_equal_eager():
             assert torch.equal(again.view(torch.int16), ref.view(torch.int16))
     with pytest.raises(RuntimeError, match="recorded for"):
         g(torch.zeros((2, 3, 1024, 1024), dtype=torch.bfloat16, device="cuda"))
+
+
+def test_derived_weight_copies_follow_load_state_dict():
+    """The K-block major weight copies and the padding-token rows are derived from module state;
+    loading other weights after a forward must not leave stale copies behind."""
+    from samfast_amd import apply_dynamic_quant
+    from samfast_amd.modeling import ImageEncoderViT
+    from samfast_amd.synthetic import init_encoder_weights, make_images
+    make = lambda: ImageEncoderViT(depth=2, embed_dim=256, num_heads=4, global_attn_indexes=(1,),
+                                   window_size=14, use_rel_pos=True, mlp_ratio=4,
+                                   norm_layer=partial(torch.nn.LayerNorm, eps=1e-6))
+    a, b = make(), make()
+    init_encoder_weights(a, seed=1)
+    init_encoder_weights(b, seed=2)
+    a = a.eval().to(torch.bfloat16).cuda()
+    b = b.eval().to(torch.bfloat16).cuda()
+    apply_dynamic_quant(a)
+    apply_dynamic_quant(b)
+    x = make_images(1, seed=4).to(torch.bfloat16).cuda()
+    with torch.no_grad():
+        ref_b = b(x).clone()
+        a(x)                                   # builds a's derived copies
+        a.load_state_dict(b.state_dict())      # in place: same storage, new values
+        out = a(x)
+    # stale copies would give an unrelated output; the neck convolutions are not run-to-run exact
+    assert _cos(out, ref_b) >= 0.9995
