@@ -100,22 +100,27 @@ struct GlobalCfg {
   static constexpr int KS = HD / 16;          // score k-steps
   static constexpr int DT = (HD + 31) / 32;   // output channel tiles
   static constexpr int BM = 128 * QT;         // queries per workgroup
-  static constexpr int KSTR = HD + 8;         // K row stride in LDS (elements)
-  static constexpr int VSTR = 64 + 8;         // V^T row stride in LDS (elements)
+  // K and V tiles travel global memory -> LDS directly (global_load_lds_dwordx4), row-major,
+  // in 16-byte pieces: a staged row is HD/8 data pieces plus one spare piece that no load
+  // writes (its lanes are masked), so rows are HD + 8 elements apart (bank spread) and 64 rows
+  // are exactly PPR wave instructions of 64 pieces.
+  static constexpr int PPR = HD / 8 + 1;      // pieces per staged row
+  static constexpr int KSTR = PPR * 8;        // K row stride in LDS (elements)
+  static constexpr int VSTR = PPR * 8;        // V row stride in LDS (elements)
   static constexpr int KBYTES = 64 * KSTR * 2;
-  // when HD is not a multiple of 32 the last output tile has spare rows: one extra V^T row of
-  // ones makes the P V product deliver the softmax denominator for free
+  static constexpr int VBYTES = 64 * VSTR * 2;
+  // when HD is not a multiple of 32 the last output tile has spare rows: the spare piece of
+  // every V row is preset to (1, 0, ..., 0), i.e. channel HD of every key is one, and the P V
+  // product delivers the softmax denominator for free
   static constexpr bool ONES_ROW = HD % 32 != 0;
-  static constexpr int VBYTES = (HD + (ONES_ROW ? 1 : 0)) * VSTR * 2;
   static constexpr int STAGE = KBYTES + VBYTES;
   static constexpr int RELH_OFF = 2 * STAGE;
   static constexpr int RELH_BYTES = 64 * BM * 4;
   static constexpr int LDS_BYTES = RELH_OFF + RELH_BYTES;
   static constexpr int XSTR = 65;             // gather scratch row stride (floats)
   static constexpr int X_BYTES = 4 * 32 * XSTR * 4;
-  static constexpr int KCH = 64 * HD / 8;     // 16-byte chunks in a K tile
-  static constexpr int KLOADS = (KCH + 255) / 256;
-  static constexpr int VBLK = 16 * (HD / 8);  // 4x8 blocks in a V tile
+  static constexpr int NDMA = PPR;            // wave instructions per K (or V) tile
+  static constexpr int DPW = (NDMA + 3) / 4;  // of which each of the 4 waves issues at most
   static_assert(X_BYTES <= 2 * STAGE, "gather scratch must fit in the K/V stages");
 };
 
@@ -142,48 +147,58 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
   const unsigned short* vbase = a.v + b * a.v_sb + h * a.v_sh;
   const unsigned short* qbase = a.q + b * a.q_sb + h * a.q_sh;
 
-  // ---- staging registers for one K/V tile ----------------------------------
-  u32x4 kst[C::KLOADS];
-  u32x4 vst[4];
-  const int v_kg = tid & 15, v_dg = tid >> 4;
-  const bool v_active = tid < C::VBLK;
-  auto stage_load = [&](int kt) {
-    const int n0 = kt * 64;
+  // ---- K/V tiles: global memory -> LDS without staging registers ----------------
+  // wave instruction n of a tile fills pieces 64n .. 64n+63 of the stage; piece P is row
+  // P / PPR, 16-byte column P % PPR (the spare column stays unwritten: lane masked)
+  typedef __attribute__((address_space(1))) const void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  int koff[C::DPW], voff[C::DPW];
 #pragma unroll
-    for (int i = 0; i < C::KLOADS; ++i) {
-      const int c = tid + 256 * i;
-      if (c < C::KCH) {
-        const int row = c / (HD / 8), col = c % (HD / 8);
-        kst[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)(n0 + row) * a.k_sn + col * 8);
+  for (int m = 0; m < C::DPW; ++m) {
+    const int P = 64 * (wave_u + 4 * m) + lane;
+    const int row = P / C::PPR, col = P % C::PPR;
+    const bool ok = (wave_u + 4 * m < C::NDMA) && col < HD / 8;
+    koff[m] = ok ? row * (int)a.k_sn + col * 8 : -1;
+    voff[m] = ok ? row * (int)a.v_sn + col * 8 : -1;
+  }
+  auto stage_dma = [&](int kt, int buf) {
+    const unsigned short* kb = kbase + (int64_t)kt * 64 * a.k_sn;
+    const unsigned short* vb = vbase + (int64_t)kt * 64 * a.v_sn;
+    unsigned char* kl = lds + buf * C::STAGE + wave_u * 1024;
+#pragma unroll
+    for (int m = 0; m < C::DPW; ++m) {
+      if (wave_u + 4 * m < C::NDMA && koff[m] >= 0) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(kb + koff[m]), (lptr_t)(kl + m * 4096), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(vb + voff[m]), (lptr_t)(kl + C::KBYTES + m * 4096), 16, 0, 0);
       }
     }
-    if (v_active) {
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk)
-        vst[kk] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)(n0 + 4 * v_kg + kk) * a.v_sn + v_dg * 8);
-    }
   };
-  auto stage_store = [&](int buf) {
-    unsigned char* kl = lds + buf * C::STAGE;
-    unsigned char* vl = kl + C::KBYTES;
+  // V^T operand of the P V product through transposing LDS reads (ds_read_b64_tr_b16): in
+  // each group of 16 lanes, lane l receives as element j the l%4-th 16-bit value of the 8
+  // bytes addressed by lane 4j + l/4 of the group.  Source lane 4j + i therefore points at
+  // key j of the lane half's four keys, channels 4i .. 4i+3 of the group's 16 channels, and
+  // lane l ends up with channel l of four consecutive keys: the MFMA A operand.
+  int vrd[C::DT];
+  {
+    const int g = lane >> 4, sl = lane & 15;
+    const int key = 4 * (g >> 1) + (sl >> 2);
 #pragma unroll
-    for (int i = 0; i < C::KLOADS; ++i) {
-      const int c = tid + 256 * i;
-      if (c < C::KCH) {
-        const int row = c / (HD / 8), col = c % (HD / 8);
-        *reinterpret_cast<u32x4*>(kl + (row * C::KSTR + col * 8) * 2) = kst[i];
-      }
+    for (int dt = 0; dt < C::DT; ++dt) {
+      int d = 32 * dt + 16 * (g & 1) + 4 * (sl & 3);
+      if (d >= HD + 8) d = HD + 4;  // past the spare piece (1, 0, .., 0): its zero half
+      vrd[dt] = (key * C::VSTR + d) * 2;
     }
-    if (v_active) {
-      u32x2 t[8];
-      transpose_4x8(vst, t);
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        *reinterpret_cast<u32x2*>(vl + ((v_dg * 8 + i) * C::VSTR + 4 * v_kg) * 2) = t[i];
-    }
+  }
+  auto vt_frag = [&](const unsigned char* vl, int dt, int j) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4* trptr_t;
+    const unsigned char* p = vl + vrd[dt] + 16 * j * C::VSTR * 2;
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)p));
+    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)(p + 8 * C::VSTR * 2)));
+    const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+    return as_bf16x8(w);
   };
-
-  stage_load(0);
 
   // ---- Q^T operand: lane holds query lr of tile t, channels 16s + 8lh .. +7 ----
   bf16x8 qf[QT][C::KS];
@@ -198,9 +213,16 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
   // b1[t][nt][r]: rel_w / sm_scale for the lane's query and key column kw of the
   // score-tile layout.  relhT[kh][q]: rel_h * log2(e).
   f32x16 b1[QT][2];
-  if (FUSED) {
+  auto first_tile = [&]() {
+    if (C::ONES_ROW && tid < 128) {  // spare piece of every V row of both stages: (1, 0, .., 0)
+      const int buf = tid >> 6, row = tid & 63;
+      const u32x4 one = {0x3F80u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(lds + buf * C::STAGE + C::KBYTES + (row * C::VSTR + HD) * 2) = one;
+    }
+    stage_dma(0, 0);
+  };
+  auto relh_from_table = [&]() {
     const unsigned short* th = a.rh;
-    const unsigned short* tw = a.rw;
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
       const int qh = (q_wg + q_wave + 32 * t) >> 6;  // one grid row per 32-query tile
@@ -224,6 +246,9 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
         }
       }
     }
+  };
+  if (FUSED) {
+    const unsigned short* tw = a.rw;
     // rel_w: T[rel][q] for rel in [0,128) in two passes of 64 through LDS scratch
     float* X = reinterpret_cast<float*>(lds) + wave * 32 * C::XSTR;
 #pragma unroll
@@ -263,7 +288,11 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
         wave_lds_fence();
       }
     }
+    __syncthreads();  // every wave is done with the scratch: the stages may be filled
+    first_tile();     // in flight while rel_h is formed
+    relh_from_table();
   } else {
+    first_tile();
     const unsigned short* rhb = a.rh + b * a.rh_sb + h * a.rh_sh + (int64_t)q_wg * a.rh_sn;
     for (int idx = tid; idx < C::BM * a.gh; idx += 256) {
       const int ql = idx % C::BM, kh = idx / C::BM;
@@ -285,13 +314,8 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
         }
     }
   }
-  __syncthreads();  // scratch reads done, relhT complete
-  if (C::ONES_ROW && tid < 2 * C::VSTR) {  // the ones row of both stages (never overwritten)
-    const int buf = tid / C::VSTR, col = tid % C::VSTR;
-    *reinterpret_cast<unsigned short*>(lds + buf * C::STAGE + C::KBYTES + (HD * C::VSTR + col) * 2) = 0x3F80;
-  }
-  stage_store(0);
-  __syncthreads();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile 0 has landed
+  __syncthreads();                                   // tile 0 and relhT complete
 
   // ---- main loop over key grid rows ---------------------------------------------
   f32x16 oacc[QT][C::DT];
@@ -310,8 +334,7 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
   for (int kt = 0; kt < nkt; ++kt) {
     const unsigned char* kl = lds + (kt & 1) * C::STAGE;
     const unsigned char* vl = kl + C::KBYTES;
-    const bool more = kt + 1 < nkt;
-    if (more) stage_load(kt + 1);
+    if (kt + 1 < nkt) stage_dma(kt + 1, (kt + 1) & 1);  // that stage was last read before the barrier
 
     // S^T = K Q^T, accumulator initialised with rel_w / sm_scale
     f32x16 s[QT][2];
@@ -368,19 +391,14 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
       for (int dt = 0; dt < C::DT; ++dt) {
-        const int drow = min(32 * dt + lr, C::ONES_ROW ? HD : HD - 1);  // row HD: ones
-        const unsigned char* vp = vl + (drow * C::VSTR + 16 * j + 4 * lh) * 2;
-        const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
-        const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 16);
-        const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
-        const bf16x8 av = as_bf16x8(w);
+        const bf16x8 av = vt_frag(vl, dt, j);
 #pragma unroll
         for (int t = 0; t < QT; ++t)
           oacc[t][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, pk[t][j], oacc[t][dt], 0, 0, 0);
       }
     }
 
-    if (more) stage_store((kt + 1) & 1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile kt+1 has landed
     __syncthreads();
   }
 
@@ -801,6 +819,8 @@ static int attn_dispatch(bool fused, AttnArgs& a, int hd, int dtype, float sm_sc
              "attn_relpos: q/k/v/out must be 16-byte aligned");
   SF_REQUIRE(a.q_sn >= hd && a.k_sn >= hd && a.v_sn >= hd && a.o_sn >= hd,
              "attn_relpos: token stride smaller than head_dim");
+  if (global_path)  // tile-relative element offsets are kept in 32 bits
+    SF_REQUIRE(a.k_sn < (1 << 24) && a.v_sn < (1 << 24), "attn_relpos: k / v token stride too large");
   if (fused) {
     SF_REQUIRE(aligned16(a.rh) && aligned16(a.rw), "attn_relpos: tables must be 16-byte aligned");
   } else if (global_path) {
