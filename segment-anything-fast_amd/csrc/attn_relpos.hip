@@ -190,14 +190,26 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
       vrd[dt] = (key * C::VSTR + d) * 2;
     }
   }
-  auto vt_frag = [&](const unsigned char* vl, int dt, int j) {
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    typedef __attribute__((address_space(3))) s16x4* trptr_t;
-    const unsigned char* p = vl + vrd[dt] + 16 * j * C::VSTR * 2;
-    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)p));
-    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)(p + 8 * C::VSTR * 2)));
-    const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
-    return as_bf16x8(w);
+  // The reads are issued as inline asm: the compiler would otherwise make each of them wait
+  // for every global->LDS load in flight (the next tile), and their completion is awaited by
+  // hand (LDS operations complete in order, so "all but the youngest n" is a counter value).
+  const unsigned int lds_base = (unsigned int)(uintptr_t)((__attribute__((address_space(3))) unsigned char*)lds);
+  auto vt_issue = [&](unsigned int stage_addr, auto jc, u32x2 (&f)[2 * C::DT]) {
+    constexpr int j = decltype(jc)::value;
+#pragma unroll
+    for (int dt = 0; dt < C::DT; ++dt) {
+      const unsigned int addr = stage_addr + vrd[dt];
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(f[2 * dt]) : "v"(addr), "n"(C::KBYTES + 16 * j * C::VSTR * 2) : "memory");
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(f[2 * dt + 1]) : "v"(addr), "n"(C::KBYTES + (16 * j + 8) * C::VSTR * 2) : "memory");
+    }
+  };
+  // all LDS operations of this wave except the youngest KEEP are complete; f is valid after it
+  auto vt_wait = [&](auto keepc, u32x2 (&f)[2 * C::DT]) {
+    constexpr int KEEP = decltype(keepc)::value;
+    if constexpr (C::DT == 3)
+      asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]) : "n"(KEEP));
+    else
+      asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]) : "n"(KEEP));
   };
 
   // ---- Q^T operand: lane holds query lr of tile t, channels 16s + 8lh .. +7 ----
@@ -332,11 +344,11 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
 
   const int nkt = a.N / 64;
   for (int kt = 0; kt < nkt; ++kt) {
-    const unsigned char* kl = lds + (kt & 1) * C::STAGE;
-    const unsigned char* vl = kl + C::KBYTES;
+    const unsigned int v_stage = lds_base + (kt & 1) * C::STAGE;
     if (kt + 1 < nkt) stage_dma(kt + 1, (kt + 1) & 1);  // that stage was last read before the barrier
 
     // S^T = K Q^T, accumulator initialised with rel_w / sm_scale
+    const unsigned char* kl = lds + (kt & 1) * C::STAGE;
     f32x16 s[QT][2];
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) {
@@ -350,6 +362,13 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
           s[t][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[t][ks], ks == 0 ? b1[t][nt] : s[t][nt], 0, 0, 0);
       }
     }
+
+    // the V^T fragments of the first two key steps travel under the softmax
+    using std::integral_constant;
+    constexpr int NF = 2 * C::DT;
+    u32x2 vf[2][NF];
+    vt_issue(v_stage, integral_constant<int, 0>{}, vf[0]);
+    vt_issue(v_stage, integral_constant<int, 1>{}, vf[1]);
 
     // online softmax, one query per lane
     bf16x8 pk[QT][4];
@@ -386,16 +405,28 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
       for (int j = 0; j < 4; ++j) pk[t][j] = cvt_bf16x8(s[t][j >> 1], 8 * (j & 1));
     }
 
-    // O^T += V^T P^T
+    // O^T += V^T P^T, the V^T fragments of key step j+1 in flight under the MFMAs of step j
+    {
+      auto pv_step = [&](auto jc, u32x2 (&f)[2 * C::DT]) {
+        constexpr int j = decltype(jc)::value;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+        for (int dt = 0; dt < C::DT; ++dt) {
+          const u32x4 w = {f[2 * dt][0], f[2 * dt][1], f[2 * dt + 1][0], f[2 * dt + 1][1]};
 #pragma unroll
-      for (int dt = 0; dt < C::DT; ++dt) {
-        const bf16x8 av = vt_frag(vl, dt, j);
-#pragma unroll
-        for (int t = 0; t < QT; ++t)
-          oacc[t][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, pk[t][j], oacc[t][dt], 0, 0, 0);
-      }
+          for (int t = 0; t < QT; ++t)
+            oacc[t][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(w), pk[t][j], oacc[t][dt], 0, 0, 0);
+        }
+      };
+      vt_wait(integral_constant<int, NF>{}, vf[0]);
+      pv_step(integral_constant<int, 0>{}, vf[0]);
+      vt_issue(v_stage, integral_constant<int, 2>{}, vf[0]);
+      vt_wait(integral_constant<int, NF>{}, vf[1]);
+      pv_step(integral_constant<int, 1>{}, vf[1]);
+      vt_issue(v_stage, integral_constant<int, 3>{}, vf[1]);
+      vt_wait(integral_constant<int, NF>{}, vf[0]);
+      pv_step(integral_constant<int, 2>{}, vf[0]);
+      vt_wait(integral_constant<int, 0>{}, vf[1]);
+      pv_step(integral_constant<int, 3>{}, vf[1]);
     }
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile kt+1 has landed
