@@ -478,14 +478,19 @@ struct WindowCfg {
   static constexpr int NT = 7;                 // key tiles of 32
   static constexpr int WAVES = 8;
   static constexpr int THREADS = 64 * WAVES;
-  static constexpr int KSTR = HD + 8;
-  static constexpr int VSTR = NMAX + 4;
+  // K and V rows travel global memory -> LDS directly, row-major, in 16-byte pieces; a staged
+  // row is HD/8 data pieces and one spare piece that no load writes (rows HD + 8 elements apart)
+  static constexpr int PPR = HD / 8 + 1;
+  static constexpr int KSTR = PPR * 8;
+  static constexpr int VSTR = PPR * 8;
   static constexpr int KBYTES = NMAX * KSTR * 2;
-  static constexpr int VBYTES = HD * VSTR * 2;
+  static constexpr int VBYTES = NMAX * VSTR * 2;
+  static constexpr int NDMA = (NMAX * PPR + 63) / 64;        // wave instructions per K (or V) window
+  static constexpr int DPW = (NDMA + WAVES - 1) / WAVES;     // of which each wavefront issues at most
   static constexpr int XSTR = 34;              // bf16 elements per scratch row
-  static constexpr int XBYTES_WAVE = 32 * XSTR * 2;  // gather scratch, aliases the K area before K is stored
+  static constexpr int XBYTES_WAVE = 32 * XSTR * 2;  // gather scratch, aliases the V area before V arrives
   static constexpr int LDS_BYTES = KBYTES + VBYTES;
-  static_assert(WAVES * XBYTES_WAVE <= KBYTES, "gather scratch must fit in the K area");
+  static_assert(WAVES * XBYTES_WAVE <= VBYTES, "gather scratch must fit in the V area");
   static_assert(NT <= WAVES, "one query tile per wavefront");
 };
 
@@ -557,36 +562,28 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
 #pragma unroll
     for (int s = 0; s < C::KS; ++s) qf[s] = load_bf16x8_global(qp + 16 * s);
   }
-  constexpr int KCH = (C::NMAX * (HD / 8) + C::THREADS - 1) / C::THREADS;            // 16-byte K chunks per thread
-  constexpr int VBL = 1;  // 4x8 V blocks per thread in the pipelined pass (196 keys x 80: 490 blocks)
-  const int nch = N * (HD / 8);
-  const int nkg_real = (N + 3) / 4;     // key groups of 4 that hold real keys
-  const int nkg = 4 * ((N + 15) / 16);  // key groups up to the 16-key step boundary: the rest is zeros
-  const int nblk = nkg_real * (HD / 8);
-  u32x4 kreg[KCH];
-  u32x4 vreg[VBL][4];
+  // wave instruction i of the window fills pieces 64i .. 64i+63: piece P is key P / PPR,
+  // 16-byte column P % PPR (spare column and keys >= N: lane masked).  K goes first and travels
+  // under the bias prologue; V follows once the scratch in its area is free.
+  typedef __attribute__((address_space(1))) const void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  auto window_dma = [&](const unsigned short* base, int64_t sn, const unsigned short* pad, unsigned char* dst) {
 #pragma unroll
-  for (int i = 0; i < KCH; ++i) {
-    const int c = min(tid + C::THREADS * i, nch - 1);
-    const int row = c / (HD / 8), col = c % (HD / 8);
-    const int tok = tok_of(row);
-    const unsigned short* src = tok >= 0 ? kbase + (int64_t)tok * a.k_sn : kpad;
-    kreg[i] = *reinterpret_cast<const u32x4*>(src + col * 8);
-  }
-#pragma unroll
-  for (int i = 0; i < VBL; ++i) {
-    const int blk = min(tid + C::THREADS * i, nblk - 1);
-    const int kg = blk / (HD / 8), dg = blk % (HD / 8);  // lanes walk along a V row: coalesced
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const int key = 4 * kg + kk;
-      const int tok = tok_of(min(key, N - 1));
-      const unsigned short* src = tok >= 0 ? vbase + (int64_t)tok * a.v_sn : vpad;
-      const u32x4 w = *reinterpret_cast<const u32x4*>(src + dg * 8);
-      const u32x4 z = {0u, 0u, 0u, 0u};
-      vreg[i][kk] = key < N ? w : z;
+    for (int m = 0; m < C::DPW; ++m) {
+      const int inst = wave_u + C::WAVES * m;
+      if (64 * inst < N * C::PPR) {  // uniform
+        const int P = 64 * inst + lane;
+        const int row = P / C::PPR, col = P % C::PPR;
+        if (row < N && col < HD / 8) {
+          const int tok = tok_of(row);
+          const unsigned short* src = (tok >= 0 ? base + (int64_t)tok * sn : pad) + col * 8;
+          __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + inst * 1024), 16, 0, 0);
+        }
+      }
     }
-  }
+  };
+  window_dma(kbase, a.k_sn, kpad, kl);
 
   // ---- bias operands while the staging loads are in flight: lane (query, lh) element e <->
   //      slot 8*lh + e.  The gather scratch lives where K will be stored afterwards ----------
@@ -595,7 +592,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     const int qh = div_gw(qc), qw = qc - qh * a.gw;
     unsigned int bhw[4] = {0u, 0u, 0u, 0u}, bww[4] = {0u, 0u, 0u, 0u};
     if (FUSED) {
-      unsigned short* X = reinterpret_cast<unsigned short*>(lds + wave * C::XBYTES_WAVE);
+      unsigned short* X = reinterpret_cast<unsigned short*>(vl + wave * C::XBYTES_WAVE);
 #pragma unroll
       for (int which = 0; which < 2; ++which) {
         // T[rel][q] = <table[rel], q> for rel in [0, 32): one MFMA row tile, staged through the
@@ -658,56 +655,44 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     bias_hv = bhv;
     bias_wv = bwv;
   }
-  __syncthreads();  // every wavefront is done with the scratch: K may overwrite it
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's share of K has landed
+  __syncthreads();  // K complete; every wavefront is done with the scratch: V may overwrite it
+  window_dma(vbase, a.v_sn, vpad, vl);
+  // V rows past the last key, up to the 16-key step boundary, are multiplied by P = 0: zeros
+  for (int idx = tid; idx < (16 * nsteps - N) * (HD / 8); idx += C::THREADS) {
+    const int row = N + idx / (HD / 8), col = idx % (HD / 8);
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    *reinterpret_cast<u32x4*>(vl + (row * C::VSTR + col * 8) * 2) = z;
+  }
+  if (!has_tile) {  // the eighth wavefront only helps with the staging
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    return;
+  }
 
-  // ---- K rows -> LDS; V 4x8 blocks -> transposed LDS (zero beyond N) ----------------------
+  // V^T operand through transposing LDS reads (ds_read_b64_tr_b16): in each group of 16 lanes,
+  // lane l receives as element j the l%4-th 16-bit value of the 8 bytes addressed by lane
+  // 4j + l/4.  Source lane 4j + i points at key j of the lane half's four keys, channels
+  // 4i .. 4i+3 of the group's 16 channels; lane l ends up with channel l of four keys.
+  int vrd[C::DT];
+  {
+    const int g = lane >> 4, sl = lane & 15;
+    const int key = 4 * (g >> 1) + (sl >> 2);
 #pragma unroll
-  for (int i = 0; i < KCH; ++i) {
-    const int c = tid + C::THREADS * i;
-    if (c < nch) {
-      const int row = c / (HD / 8), col = c % (HD / 8);
-      *reinterpret_cast<u32x4*>(kl + (row * C::KSTR + col * 8) * 2) = kreg[i];
+    for (int dt = 0; dt < C::DT; ++dt) {
+      const int d = min(32 * dt + 16 * (g & 1) + 4 * (sl & 3), HD - 4);  // rows >= HD of the last tile: unused
+      vrd[dt] = (key * C::VSTR + d) * 2;
     }
   }
-#pragma unroll
-  for (int i = 0; i < VBL; ++i) {
-    const int blk = tid + C::THREADS * i;
-    if (blk < nblk) {
-      const int kg = blk / (HD / 8), dg = blk % (HD / 8);
-      u32x2 t[8];
-      transpose_4x8(vreg[i], t);
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        *reinterpret_cast<u32x2*>(vl + ((dg * 8 + j) * C::VSTR + 4 * kg) * 2) = t[j];
-    }
-  }
-  // blocks beyond one per thread (windows of more than 204 tokens only): plain load-store pass
-  for (int blk = tid + C::THREADS * VBL; blk < nblk; blk += C::THREADS) {
-    const int kg = blk / (HD / 8), dg = blk % (HD / 8);
-    u32x4 in[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const int key = 4 * kg + kk;
-      const int tok = tok_of(min(key, N - 1));
-      const unsigned short* src = tok >= 0 ? vbase + (int64_t)tok * a.v_sn : vpad;
-      const u32x4 w = *reinterpret_cast<const u32x4*>(src + dg * 8);
-      const u32x4 z = {0u, 0u, 0u, 0u};
-      in[kk] = key < N ? w : z;
-    }
-    u32x2 t[8];
-    transpose_4x8(in, t);
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-      *reinterpret_cast<u32x2*>(vl + ((dg * 8 + j) * C::VSTR + 4 * kg) * 2) = t[j];
-  }
-  // key groups past the last real key, up to the 16-key step boundary: zeros
-  for (int idx = tid; idx < (nkg - nkg_real) * HD; idx += C::THREADS) {
-    const int kg = nkg_real + idx / HD, d = idx % HD;
-    const u32x2 z = {0u, 0u};
-    *reinterpret_cast<u32x2*>(vl + (d * C::VSTR + 4 * kg) * 2) = z;
-  }
-  __syncthreads();
-  if (!has_tile) return;  // the eighth wavefront only helps with the staging
+  auto vt_frag = [&](int dt, int j) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4* trptr_t;
+    const unsigned char* p = vl + vrd[dt] + 16 * j * C::VSTR * 2;
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)p));
+    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)(p + 8 * C::VSTR * 2)));
+    const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+    return as_bf16x8(w);
+  };
 
   const bf16x8 bh_op = as_bf16x8(bias_hv), bw_op = as_bf16x8(bias_wv);
 
@@ -754,7 +739,10 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
         lsum += p;
       }
       l_run = l_run * alpha + lsum;
-      if (__any(alpha != 1.0f)) {
+      if (nt == 0) {  // V travelled under the first score tile; every wavefront's share has landed
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+      } else if (__any(alpha != 1.0f)) {
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
@@ -767,12 +755,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
           const bf16x8 pk = cvt_bf16x8(acc, 8 * half);
 #pragma unroll
           for (int dt = 0; dt < C::DT; ++dt) {
-            const int drow = min(32 * dt + lr, HD - 1);
-            const unsigned char* vp = vl + (drow * C::VSTR + 16 * j + 4 * lh) * 2;
-            const u32x2 lo = *reinterpret_cast<const u32x2*>(vp);
-            const u32x2 hi = *reinterpret_cast<const u32x2*>(vp + 16);
-            const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
-            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(w), pk, oacc[dt], 0, 0, 0);
+            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt_frag(dt, j), pk, oacc[dt], 0, 0, 0);
           }
         }
       }
