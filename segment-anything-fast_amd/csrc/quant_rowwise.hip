@@ -107,13 +107,18 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
   }
   const u32x4* src = reinterpret_cast<const u32x4*>(a.x + srow * a.ldx);
 
-  u32x4 buf[NCH];
+  // the row as floats, unpacked once: lane holds chunks lane, lane + 64, ... of 8 elements
+  float f[NCH][8];
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = lane + i * 64;
     u32x4 w = {0u, 0u, 0u, 0u};
     if (c < nchunk) w = src[c];
-    buf[i] = w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[i][2 * j] = bf16_lo_to_f32(w[j]);
+      f[i][2 * j + 1] = bf16_hi_to_f32(w[j]);
+    }
   }
 
   if (LN) {
@@ -122,7 +127,7 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
 #pragma unroll
     for (int i = 0; i < NCH; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) s1 += bf16_lo_to_f32(buf[i][j]) + bf16_hi_to_f32(buf[i][j]);
+      for (int j = 0; j < 4; ++j) s1 += f[i][2 * j] + f[i][2 * j + 1];
     const float mean = wave_sum(s1) / (float)a.K;
     float s2 = 0.f;
 #pragma unroll
@@ -130,7 +135,9 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
       if (lane + i * 64 < nchunk) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float d0 = bf16_lo_to_f32(buf[i][j]) - mean, d1 = bf16_hi_to_f32(buf[i][j]) - mean;
+          const float d0 = f[i][2 * j] - mean, d1 = f[i][2 * j + 1] - mean;
+          f[i][2 * j] = d0;
+          f[i][2 * j + 1] = d1;
           s2 += d0 * d0 + d1 * d1;
         }
       }
@@ -145,9 +152,11 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
         const u32x4 g = g4[c], b = b4[c];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float y0 = (bf16_lo_to_f32(buf[i][j]) - mean) * rstd * bf16_lo_to_f32(g[j]) + bf16_lo_to_f32(b[j]);
-          const float y1 = (bf16_hi_to_f32(buf[i][j]) - mean) * rstd * bf16_hi_to_f32(g[j]) + bf16_hi_to_f32(b[j]);
-          buf[i][j] = pack_bf16x2(y0, y1);  // the bf16 value a separate LayerNorm would have stored
+          const float y0 = f[i][2 * j] * rstd * bf16_lo_to_f32(g[j]) + bf16_lo_to_f32(b[j]);
+          const float y1 = f[i][2 * j + 1] * rstd * bf16_hi_to_f32(g[j]) + bf16_hi_to_f32(b[j]);
+          const unsigned int y = pack_bf16x2(y0, y1);  // the bf16 values a separate LayerNorm would have stored
+          f[i][2 * j] = bf16_lo_to_f32(y);
+          f[i][2 * j + 1] = bf16_hi_to_f32(y);
         }
       }
     }
@@ -157,10 +166,7 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
 #pragma unroll
   for (int i = 0; i < NCH; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      amax = fmaxf(amax, fabsf(bf16_lo_to_f32(buf[i][j])));
-      amax = fmaxf(amax, fabsf(bf16_hi_to_f32(buf[i][j])));
-    }
+    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(f[i][e]));
   amax = wave_max(amax);
 
   const float scale = fmaxf(amax, 1e-5f) / 127.0f;
@@ -170,15 +176,7 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = lane + i * 64;
-    if (c < nchunk) {
-      float v[8];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        v[2 * j] = bf16_lo_to_f32(buf[i][j]);
-        v[2 * j + 1] = bf16_hi_to_f32(buf[i][j]);
-      }
-      *dst_of(c) = quantize8(v, scale, inv_scale);
-    }
+    if (c < nchunk) *dst_of(c) = quantize8(f[i], scale, inv_scale);
   }
 }
 
