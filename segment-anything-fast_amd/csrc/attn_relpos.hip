@@ -63,6 +63,7 @@ struct AttnArgs {
 };
 
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLazyLog2 = 8.0f;  // softmax reference lags the running maximum by at most 2^8
 
 SF_DEVICE bf16x8 as_bf16x8(u32x4 w) { return __builtin_bit_cast(bf16x8, w); }
 
@@ -381,10 +382,21 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[t][1][r]);
       mx = fmaxf(mx, xor32(mx));
       const float b0 = relhT[kt * C::BM + q_wave + 32 * t + lr];
+      // lazy reference: the exponent offset m_i follows the running maximum only when that has
+      // grown by more than kLazyLog2 (p stays <= 2^kLazyLog2; the final division by the
+      // denominator, accumulated with the same offsets, makes the result independent of it),
+      // so the accumulators are rescaled a few times per row of keys instead of once per tile
       const float m_new = fmaxf(m_i[t], fmaf(mx, a.c, b0));
-      const float alpha = fast_exp2(m_i[t] - m_new);
-      m_i[t] = m_new;
-      const float neg_mrow = b0 - m_new;
+      float alpha = 1.0f;
+      if (__any(m_new - m_i[t] > kLazyLog2)) {  // uniform; first tile: m_i = -inf
+        alpha = fast_exp2(m_i[t] - m_new);
+        m_i[t] = m_new;
+#pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[t][dt][r] *= alpha;
+      }
+      const float neg_mrow = b0 - m_i[t];
       float lsum = 0.f;
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
@@ -395,12 +407,6 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
           if (!C::ONES_ROW) lsum += p;
         }
       if (!C::ONES_ROW) l_i[t] = l_i[t] * alpha + lsum;
-      if (__any(alpha != 1.0f)) {
-#pragma unroll
-        for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[t][dt][r] *= alpha;
-      }
 #pragma unroll
       for (int j = 0; j < 4; ++j) pk[t][j] = cvt_bf16x8(s[t][j >> 1], 8 * (j & 1));
     }
@@ -727,10 +733,15 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
 #pragma unroll
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, acc[r]);
       mx = fmaxf(mx, xor32(mx));
+      // lazy reference (see the global kernel): m_run follows the maximum in steps > 2^kLazyLog2
       const float m_new = fmaxf(m_run, mx);
-      const float alpha = fast_exp2((m_run - m_new) * a.c);
-      const float neg_m = -m_new * a.c;
-      m_run = m_new;
+      float alpha = 1.0f;
+      const bool move = __any((m_new - m_run) * a.c > kLazyLog2);  // uniform; first tile: always
+      if (move) {
+        alpha = fast_exp2((m_run - m_new) * a.c);
+        m_run = m_new;
+      }
+      const float neg_m = -m_run * a.c;
       float lsum = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -742,7 +753,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
       if (nt == 0) {  // V travelled under the first score tile; every wavefront's share has landed
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-      } else if (__any(alpha != 1.0f)) {
+      } else if (move) {
 #pragma unroll
         for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
