@@ -493,6 +493,9 @@ struct WindowCfg {
   static constexpr int VBYTES = NMAX * VSTR * 2;
   static constexpr int NDMA = (NMAX * PPR + 63) / 64;        // wave instructions per K (or V) window
   static constexpr int DPW = (NDMA + WAVES - 1) / WAVES;     // of which each wavefront issues at most
+  // when HD is not a multiple of 32 the last output tile has spare rows: the spare piece of
+  // every V row is preset to (1, 0, ..., 0) and row HD of O^T is the softmax denominator
+  static constexpr bool ONES_ROW = HD % 32 != 0;
   static constexpr int XSTR = 34;              // bf16 elements per scratch row
   static constexpr int XBYTES_WAVE = 32 * XSTR * 2;  // gather scratch, aliases the V area before V arrives
   static constexpr int LDS_BYTES = KBYTES + VBYTES;
@@ -574,18 +577,22 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
   typedef __attribute__((address_space(1))) const void* gptr_t;
   typedef __attribute__((address_space(3))) void* lptr_t;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  // per issued instruction: the lane's token row (-1 padding token, -2 lane masked) and column
+  int dma_tok[C::DPW], dma_col[C::DPW];
+#pragma unroll
+  for (int m = 0; m < C::DPW; ++m) {
+    const int P = 64 * (wave_u + C::WAVES * m) + lane;
+    const int row = P / C::PPR, col = P % C::PPR;
+    dma_col[m] = col * 8;
+    dma_tok[m] = (row < N && col < HD / 8) ? tok_of(row) : -2;
+  }
   auto window_dma = [&](const unsigned short* base, int64_t sn, const unsigned short* pad, unsigned char* dst) {
 #pragma unroll
     for (int m = 0; m < C::DPW; ++m) {
       const int inst = wave_u + C::WAVES * m;
-      if (64 * inst < N * C::PPR) {  // uniform
-        const int P = 64 * inst + lane;
-        const int row = P / C::PPR, col = P % C::PPR;
-        if (row < N && col < HD / 8) {
-          const int tok = tok_of(row);
-          const unsigned short* src = (tok >= 0 ? base + (int64_t)tok * sn : pad) + col * 8;
-          __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + inst * 1024), 16, 0, 0);
-        }
+      if (64 * inst < N * C::PPR && dma_tok[m] > -2) {  // first test uniform
+        const unsigned short* src = (dma_tok[m] >= 0 ? base + (int64_t)dma_tok[m] * sn : pad) + dma_col[m];
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + inst * 1024), 16, 0, 0);
       }
     }
   };
@@ -670,6 +677,10 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     const u32x4 z = {0u, 0u, 0u, 0u};
     *reinterpret_cast<u32x4*>(vl + (row * C::VSTR + col * 8) * 2) = z;
   }
+  if (C::ONES_ROW && tid < 16 * nsteps) {  // the ones channel (P = 0 beyond the last key anyway)
+    const u32x4 one = {0x3F80u, 0u, 0u, 0u};
+    *reinterpret_cast<u32x4*>(vl + (tid * C::VSTR + HD) * 2) = one;
+  }
   if (!has_tile) {  // the eighth wavefront only helps with the staging
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -686,7 +697,9 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     const int key = 4 * (g >> 1) + (sl >> 2);
 #pragma unroll
     for (int dt = 0; dt < C::DT; ++dt) {
-      const int d = min(32 * dt + 16 * (g & 1) + 4 * (sl & 3), HD - 4);  // rows >= HD of the last tile: unused
+      int d = 32 * dt + 16 * (g & 1) + 4 * (sl & 3);
+      if (C::ONES_ROW) d = d >= HD + 8 ? HD + 4 : d;  // past the spare piece (1, 0, .., 0): its zero half
+      else d = min(d, HD - 4);
       vrd[dt] = (key * C::VSTR + d) * 2;
     }
   }
@@ -747,9 +760,9 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
       for (int r = 0; r < 16; ++r) {
         const float p = fast_exp2(fmaf(acc[r], a.c, neg_m));
         acc[r] = p;
-        lsum += p;
+        if (!C::ONES_ROW) lsum += p;
       }
-      l_run = l_run * alpha + lsum;
+      if (!C::ONES_ROW) l_run = l_run * alpha + lsum;
       if (nt == 0) {  // V travelled under the first score tile; every wavefront's share has landed
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -772,7 +785,17 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
       }
     }
   }
-  const float l = l_run + xor32(l_run);
+  float l;
+  if (C::ONES_ROW) {
+    // output row HD = tile DT-1, row HD % 32, held by the lh = (HD % 32) / 4 % 2 lanes
+    constexpr int orow = HD % 32;
+    constexpr int oreg = 4 * (orow / 8) + orow % 4, olh = (orow / 4) % 2;
+    const float own = oacc[C::DT - 1][oreg];
+    const float other = xor32(own);
+    l = (lh == olh) ? own : other;
+  } else {
+    l = l_run + xor32(l_run);
+  }
   const float inv = 1.0f / l;
   const int otok = qi < N ? tok_of(qi) : -1;  // padding queries produce no output
   if (otok >= 0) {
