@@ -178,3 +178,27 @@ def test_windowed_on_image_tokens_equals_partitioned_windows(B, nH, H, W, ws, hd
     ref = ora.window_unpartition(ref, ws, (Hp, Wp), (H, W)).reshape(B, H * W, nH, hd)
     err = (out.float().cpu() - ref).abs()
     assert err.max() <= 2e-2 and err.mean() <= 1e-3, (err.max(), err.mean())
+
+
+@pytest.mark.parametrize("gh,gw,hd,ramp", [(64, 64, 80, 0.02), (64, 64, 64, 3.0), (14, 14, 80, 0.5), (14, 14, 64, 6.0)])
+def test_rising_maximum_along_the_keys(gh, gw, hd, ramp):
+    """The kernels rescale their accumulators only when the running maximum has grown by more than
+    2^8 since the last rescale.  Keys whose logits rise steadily with the key index make the
+    maximum move in every tile: slowly (never past the threshold after the first tile) or fast
+    (past it every few tiles); both must agree with the oracle."""
+    from samfast_amd import ops
+    B, nH = 1, 2
+    N = gh * gw
+    q, k, v, rph, rpw = attn_inputs(B, nH, gh, gw, hd, seed=7)
+    # one shared direction u: q gets a positive component along u, key n the component ramp*n/N*|u|
+    g = torch.Generator().manual_seed(3)
+    u = torch.randn(hd, generator=g)
+    u = u / u.norm()
+    steps = torch.arange(N, dtype=torch.float32) / N
+    q = (q.float() + 4.0 * u).to(torch.bfloat16)
+    k = (k.float() + (ramp * math.sqrt(hd) * 8.0) * steps[None, None, :, None] * u).to(torch.bfloat16)
+    ref = _oracle_tables(q, k, v, rph, rpw, (gh, gw))
+    dev = "cuda"
+    out = ops.attn_relpos(q.to(dev), k.to(dev), v.to(dev), rph.to(dev), rpw.to(dev), (gh, gw))
+    torch.cuda.synchronize()
+    _check(out, ref, f"rising max {gh}x{gw}x{hd} ramp {ramp}")
