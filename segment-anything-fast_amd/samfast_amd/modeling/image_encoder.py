@@ -351,4 +351,15 @@ class PatchEmbed(nn.Module):
                               padding=padding)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        p = self.proj
+        kh, kw = p.kernel_size
+        if (x.is_cuda and p.stride == p.kernel_size and p.padding == (0, 0) and p.dilation == (1, 1)
+                and p.groups == 1 and x.shape[2] % kh == 0 and x.shape[3] % kw == 0):
+            # non-overlapping patches: the convolution is one GEMM over (channel, dy, dx) whose
+            # output is already (B, H, W, C)
+            B, C, H, W = x.shape
+            gh, gw = H // kh, W // kw
+            cols = x.view(B, C, gh, kh, gw, kw).permute(0, 2, 4, 1, 3, 5).reshape(B * gh * gw, C * kh * kw)
+            y = F.linear(cols, p.weight.view(p.out_channels, C * kh * kw), p.bias)
+            return y.view(B, gh, gw, p.out_channels)
         return self.proj(x).permute(0, 2, 3, 1)
