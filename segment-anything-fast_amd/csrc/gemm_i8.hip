@@ -187,6 +187,9 @@ SF_DEVICE void gemm_epilogue_staged(const GemmArgs& a, i32x16 (&acc)[2][4], unsi
   const int chunk = tid & 31, rsub = tid >> 5;
   const int n = n0 + chunk * 8;
   const bool col_ok = n < a.N;  // N % 8 == 0
+  // a tile that lies inside the matrix and is not row-scattered takes straight-line code: no
+  // predicates, so all residual loads and all tile reads of phase 2 are in flight together
+  const bool full = m0 + 128 <= a.M && n0 + GBN <= a.N && !(EPI == EPI_RESIDUAL_BF16 && a.dst_row);
   auto out_row = [&](int p) {
     const int row = 8 * p + rsub;
     if (m0 + row >= a.M || !col_ok) return -1;
@@ -198,12 +201,18 @@ SF_DEVICE void gemm_epilogue_staged(const GemmArgs& a, i32x16 (&acc)[2][4], unsi
   // their latency is hidden behind it
   u32x4 res[16];
   if (EPI == EPI_RESIDUAL_BF16) {
+    if (full) {
+      const unsigned short* rp = a.residual + (int64_t)(m0 + rsub) * a.ld_res + n;
 #pragma unroll
-    for (int p = 0; p < 16; ++p) {
-      const u32x4 z = {0u, 0u, 0u, 0u};
-      res[p] = z;
-      const int dr = out_row(p);
-      if (dr >= 0) res[p] = *reinterpret_cast<const u32x4*>(a.residual + (int64_t)dr * a.ld_res + n);
+      for (int p = 0; p < 16; ++p) res[p] = *reinterpret_cast<const u32x4*>(rp + (int64_t)(8 * p) * a.ld_res);
+    } else {
+#pragma unroll
+      for (int p = 0; p < 16; ++p) {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        res[p] = z;
+        const int dr = out_row(p);
+        if (dr >= 0) res[p] = *reinterpret_cast<const u32x4*>(a.residual + (int64_t)dr * a.ld_res + n);
+      }
     }
   }
 
@@ -246,18 +255,32 @@ SF_DEVICE void gemm_epilogue_staged(const GemmArgs& a, i32x16 (&acc)[2][4], unsi
   __builtin_amdgcn_sched_barrier(0);
 
   unsigned short* outp = reinterpret_cast<unsigned short*>(a.out);
+  const unsigned char* tile = lds + rsub * EP_STRIDE + chunk * 16;
+  auto add_residual = [&](u32x4& val, const u32x4& r) {
 #pragma unroll
-  for (int p = 0; p < 16; ++p) {
-    const int dr = out_row(p);
-    u32x4 val = *reinterpret_cast<const u32x4*>(lds + (8 * p + rsub) * EP_STRIDE + chunk * 16);
-    if (EPI == EPI_RESIDUAL_BF16) {
+    for (int c = 0; c < 4; ++c)
+      // bf16 add of the bf16-rounded Linear output and the residual stream
+      val[c] = pack_bf16x2(bf16_lo_to_f32(val[c]) + bf16_lo_to_f32(r[c]),
+                           bf16_hi_to_f32(val[c]) + bf16_hi_to_f32(r[c]));
+  };
+  if (full) {
+    u32x4 val[16];
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        // bf16 add of the bf16-rounded Linear output and the residual stream
-        val[c] = pack_bf16x2(bf16_lo_to_f32(val[c]) + bf16_lo_to_f32(res[p][c]),
-                             bf16_hi_to_f32(val[c]) + bf16_hi_to_f32(res[p][c]));
+    for (int p = 0; p < 16; ++p) val[p] = *reinterpret_cast<const u32x4*>(tile + 8 * p * EP_STRIDE);
+    unsigned short* op = outp + (int64_t)(m0 + rsub) * a.ldo + n;
+#pragma unroll
+    for (int p = 0; p < 16; ++p) {
+      if (EPI == EPI_RESIDUAL_BF16) add_residual(val[p], res[p]);
+      *reinterpret_cast<u32x4*>(op + (int64_t)(8 * p) * a.ldo) = val[p];
     }
-    if (dr >= 0) *reinterpret_cast<u32x4*>(outp + (int64_t)dr * a.ldo + n) = val;
+  } else {
+#pragma unroll
+    for (int p = 0; p < 16; ++p) {
+      const int dr = out_row(p);
+      u32x4 val = *reinterpret_cast<const u32x4*>(tile + 8 * p * EP_STRIDE);
+      if (EPI == EPI_RESIDUAL_BF16) add_residual(val, res[p]);
+      if (dr >= 0) *reinterpret_cast<u32x4*>(outp + (int64_t)dr * a.ldo + n) = val;
+    }
   }
 }
 
