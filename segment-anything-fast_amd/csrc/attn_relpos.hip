@@ -9,8 +9,12 @@
 // r%4), so the softmax row statistics are per-lane scalars: the row maximum and
 // sum are reduced in registers plus one exchange with lane^32.  The same
 // registers, converted to bf16, are directly the B operand (P^T) of the second
-// product O^T = V^T P^T, whose A operand is read from a transposed copy of V in
-// LDS with two 8-byte reads that follow the key order of the P registers.
+// product O^T = V^T P^T.  K and V tiles travel global memory -> LDS directly
+// (global_load_lds_dwordx4), row-major; the V^T operand is formed by transposing
+// LDS reads (ds_read_b64_tr_b16) that follow the key order of the P registers.
+// The exponent offset of the online softmax follows the running maximum lazily
+// (only in steps of more than 2^8), so the output accumulators are rescaled a
+// few times per row of keys instead of once per key tile.
 //
 // Everything runs in the base-2 domain with the exact scale folded into the
 // exponent argument: p = exp2(fma(s, c, -m)), c = sm_scale*log2(e), so q is
@@ -80,18 +84,6 @@ SF_DEVICE bf16x8 cvt_bf16x8(const f32x16& s, int base) {
 
 // all LDS operations this wavefront has issued are complete and ordered
 SF_DEVICE void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-
-// transpose a 4-key x 8-channel block held as 4 x 16 bytes into 8 x (4 keys) 8-byte rows
-SF_DEVICE void transpose_4x8(const u32x4 (&in)[4], u32x2 (&outv)[8]) {
-#pragma unroll
-  for (int m = 0; m < 4; ++m) {
-    const unsigned int k0 = in[0][m], k1 = in[1][m], k2 = in[2][m], k3 = in[3][m];
-    outv[2 * m][0] = (k0 & 0xffffu) | (k1 << 16);
-    outv[2 * m][1] = (k2 & 0xffffu) | (k3 << 16);
-    outv[2 * m + 1][0] = (k0 >> 16) | (k1 & 0xffff0000u);
-    outv[2 * m + 1][1] = (k2 >> 16) | (k3 & 0xffff0000u);
-  }
-}
 
 // =============================================================================
 // global kernel: gw == 64, N % (128*QT) == 0
