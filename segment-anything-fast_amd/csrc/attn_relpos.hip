@@ -82,6 +82,16 @@ SF_DEVICE bf16x8 cvt_bf16x8(const f32x16& s, int base) {
   return as_bf16x8(w);
 }
 
+// max(v, v of lane ^ 32) without an LDS round trip: v_permlane32_swap exchanges the upper half
+// of its first operand with the lower half of its second, after which every lane holds its own
+// value in one of the two and its partner's in the other
+SF_DEVICE float max_with_lane_xor32(float v) {
+  typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+  const unsigned int b = __float_as_uint(v);
+  const u32x2_t r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 // all LDS operations this wavefront has issued are complete and ordered
 SF_DEVICE void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
@@ -372,7 +382,7 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[t][0][r]);
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[t][1][r]);
-      mx = fmaxf(mx, xor32(mx));
+      mx = max_with_lane_xor32(mx);
       const float b0 = relhT[kt * C::BM + q_wave + 32 * t + lr];
       // lazy reference: the exponent offset m_i follows the running maximum only when that has
       // grown by more than kLazyLog2 (p stays <= 2^kLazyLog2; the final division by the
@@ -737,7 +747,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
       float mx = acc[0];
 #pragma unroll
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, acc[r]);
-      mx = fmaxf(mx, xor32(mx));
+      mx = max_with_lane_xor32(mx);
       // lazy reference (see the global kernel): m_run follows the maximum in steps > 2^kLazyLog2
       const float m_new = fmaxf(m_run, mx);
       float alpha = 1.0f;
