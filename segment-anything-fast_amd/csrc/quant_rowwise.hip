@@ -35,27 +35,49 @@ struct QuantArgs {
   int kb64;  // 1: write xq K-block major, (K/64, M, 64)
 };
 
-SF_DEVICE float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
+// Wavefront-wide reductions without LDS traffic: four DPP steps combine the 16 lanes of a row
+// (lane ^ 1, lane ^ 2, then the mirrored half row and the mirrored row, which by then hold the
+// other quad's / other half's partial result), two lane-swap steps combine the four rows.
+template <int CTRL>
+SF_DEVICE float dpp_f32(float v) {
+  return __uint_as_float((unsigned int)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
 }
-SF_DEVICE float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
+template <typename Op>
+SF_DEVICE float wave_reduce(float v, Op op) {
+  v = op(v, dpp_f32<0xB1>(v));   // quad_perm [1, 0, 3, 2]
+  v = op(v, dpp_f32<0x4E>(v));   // quad_perm [2, 3, 0, 1]
+  v = op(v, dpp_f32<0x141>(v));  // row_half_mirror
+  v = op(v, dpp_f32<0x140>(v));  // row_mirror
+  typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+  unsigned int b = __float_as_uint(v);
+  u32x2_t r = __builtin_amdgcn_permlane16_swap(b, b, false, false);  // rows 0<->1, 2<->3
+  v = op(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  b = __float_as_uint(v);
+  r = __builtin_amdgcn_permlane32_swap(b, b, false, false);          // halves of the wavefront
+  return op(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+SF_DEVICE float wave_sum(float v) {
+  return wave_reduce(v, [](float x, float y) { return x + y; });
+}
+// for values >= 0 (absolute maxima): the bit patterns order like the values, and the unsigned
+// maximum needs no canonicalisation of its operands
+SF_DEVICE float wave_max_nonneg(float v) {
+  return wave_reduce(v, [](float x, float y) {
+    return __uint_as_float(max(__float_as_uint(x), __float_as_uint(y)));
+  });
 }
 
-// 8 values -> 8 int8 codes packed in 8 bytes.
+// EPC (4 or 8) values -> EPC int8 codes packed in EPC bytes.
 // Rounding: adding 1.5 * 2^23 to r (|r| <= 127) leaves rint(r) - half to even - in the low
 // mantissa bits, so the low byte of the sum's bit pattern is the int8 code; subtracting the
 // constant again gives rint(r) as a float for the near-tie test.
-SF_DEVICE u32x2 quantize8(const float (&v)[8], float scale, float inv_scale) {
+template <int EPC>
+SF_DEVICE void quantize_chunk(const float (&v)[EPC], float scale, float inv_scale, unsigned int (&out)[EPC / 4]) {
   constexpr float kMagic = 12582912.0f;  // 1.5 * 2^23
-  float m[8];
+  float m[EPC];
   bool near_tie = false;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
+  for (int e = 0; e < EPC; ++e) {
     const float r = v[e] * inv_scale;
     m[e] = r + kMagic;
     const float d = r - (m[e] - kMagic);  // r - rint(r), exact
@@ -63,63 +85,91 @@ SF_DEVICE u32x2 quantize8(const float (&v)[8], float scale, float inv_scale) {
   }
   if (near_tie) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) m[e] = v[e] / scale + kMagic;  // IEEE division
+    for (int e = 0; e < EPC; ++e) m[e] = v[e] / scale + kMagic;  // IEEE division
   }
-  unsigned int b[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) b[e] = __builtin_bit_cast(unsigned int, m[e]);
-  // byte 0 of each of four words -> one word (v_perm_b32: selector bytes pick from {hi, lo})
-  auto pack4 = [](unsigned int w0, unsigned int w1, unsigned int w2, unsigned int w3) {
+  for (int g = 0; g < EPC / 4; ++g) {
+    const unsigned int w0 = __builtin_bit_cast(unsigned int, m[4 * g]), w1 = __builtin_bit_cast(unsigned int, m[4 * g + 1]);
+    const unsigned int w2 = __builtin_bit_cast(unsigned int, m[4 * g + 2]), w3 = __builtin_bit_cast(unsigned int, m[4 * g + 3]);
+    // byte 0 of each of four words -> one word (v_perm_b32: selector bytes pick from {hi, lo})
     const unsigned int lo = __builtin_amdgcn_perm(w1, w0, 0x0c0c0400u);  // [w0.b0, w1.b0, 0, 0]
     const unsigned int hi = __builtin_amdgcn_perm(w3, w2, 0x04000c0cu);  // [0, 0, w2.b0, w3.b0]
-    return lo | hi;
-  };
-  const u32x2 o = {pack4(b[0], b[1], b[2], b[3]), pack4(b[4], b[5], b[6], b[7])};
-  return o;
+    out[g] = lo | hi;
+  }
 }
 
-template <int NCH, bool LN>  // 16-byte chunks per lane: covers K <= NCH * 512
+// A lane holds chunks lane, lane + 64, ... of EPC elements (NCH of them: K <= NCH * 64 * EPC).
+// EPC = 8 (16-byte loads) is the general case; EPC = 4 (8-byte loads) is taken when it divides the
+// row among the lanes without a remainder and EPC = 8 does not (K = 1280: five chunks of 4 per
+// lane instead of three chunks of 8 of which the third is half empty).
+template <int NCH, int EPC, bool LN>
 __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_kernel(QuantArgs a) {
+  static_assert(EPC == 4 || EPC == 8, "chunk width");
+  constexpr int W = EPC / 2;  // 32-bit words per input chunk
+  typedef unsigned int in_t __attribute__((ext_vector_type(W)));
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * kQuantWavesPerBlock + (threadIdx.x >> 6);
   if (row >= a.M) return;  // whole wavefront leaves together
-  const int nchunk = a.K >> 3;
-  // 8-byte chunk c of the row: row-major at row*K + 8c; K-block major at ((c/8)*M + row)*64 + (c%8)*8
-  auto dst_of = [&](int c) {
-    const int64_t off = a.kb64 ? ((int64_t)(c >> 3) * a.M + row) * 64 + (c & 7) * 8
-                               : row * (int64_t)a.K + (int64_t)c * 8;
-    return reinterpret_cast<u32x2*>(a.xq + off);
+  const int nchunk = a.K / EPC;
+  // chunk c of the row: row-major at row*K + EPC*c; K-block major at ((c*EPC/64)*M + row)*64 + (c*EPC)%64
+  auto store_chunk = [&](int c, const unsigned int (&codes)[EPC / 4]) {
+    const int k = c * EPC;
+    const int64_t off = a.kb64 ? ((int64_t)(k >> 6) * a.M + row) * 64 + (k & 63)
+                               : row * (int64_t)a.K + k;
+    unsigned int* dst = reinterpret_cast<unsigned int*>(a.xq + off);
+    if (EPC == 8) {
+      const u32x2 o = {codes[0], codes[EPC / 4 - 1]};
+      *reinterpret_cast<u32x2*>(dst) = o;
+    } else {
+      *dst = codes[0];
+    }
   };
 
   int64_t srow = row;
   if (LN && a.src_row) {
     srow = a.src_row[row];
     if (srow < 0) {  // a padding token: LayerNorm output replaced by zeros
-      const u32x2 z = {0u, 0u};
+      const unsigned int z[EPC / 4] = {};
 #pragma unroll
       for (int i = 0; i < NCH; ++i) {
         const int c = lane + i * 64;
-        if (c < nchunk) *dst_of(c) = z;
+        if (c < nchunk) store_chunk(c, z);
       }
       if (lane == 0) a.sx[row] = 1e-5f / 127.0f;
       return;
     }
   }
-  const u32x4* src = reinterpret_cast<const u32x4*>(a.x + srow * a.ldx);
+  const in_t* src = reinterpret_cast<const in_t*>(a.x + srow * a.ldx);
 
-  // the row as floats, unpacked once: lane holds chunks lane, lane + 64, ... of 8 elements
-  float f[NCH][8];
+  // all global loads first: the row, and (LN) the lane's slices of gamma and beta, which do not
+  // depend on the statistics and would otherwise add a second memory latency to the chain
+  in_t xw[NCH], gw[LN ? NCH : 1], bw[LN ? NCH : 1];
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = lane + i * 64;
-    u32x4 w = {0u, 0u, 0u, 0u};
-    if (c < nchunk) w = src[c];
+    const in_t z = {};
+    xw[i] = z;
+    if (c < nchunk) xw[i] = src[c];
+  }
+  if (LN) {
+    const in_t* g4 = reinterpret_cast<const in_t*>(a.gamma);
+    const in_t* b4 = reinterpret_cast<const in_t*>(a.beta);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      f[i][2 * j] = bf16_lo_to_f32(w[j]);
-      f[i][2 * j + 1] = bf16_hi_to_f32(w[j]);
+    for (int i = 0; i < NCH; ++i) {
+      const int c = min(lane + i * 64, nchunk - 1);
+      gw[i] = g4[c];
+      bw[i] = b4[c];
     }
   }
+  // the row as floats, unpacked once
+  float f[NCH][EPC];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      f[i][2 * j] = bf16_lo_to_f32(xw[i][j]);
+      f[i][2 * j + 1] = bf16_hi_to_f32(xw[i][j]);
+    }
 
   if (LN) {
     // two-pass mean / biased variance over the K real elements, fp32
@@ -127,14 +177,14 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
 #pragma unroll
     for (int i = 0; i < NCH; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) s1 += f[i][2 * j] + f[i][2 * j + 1];
+      for (int j = 0; j < W; ++j) s1 += f[i][2 * j] + f[i][2 * j + 1];
     const float mean = wave_sum(s1) / (float)a.K;
     float s2 = 0.f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       if (lane + i * 64 < nchunk) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < W; ++j) {
           const float d0 = f[i][2 * j] - mean, d1 = f[i][2 * j + 1] - mean;
           f[i][2 * j] = d0;
           f[i][2 * j + 1] = d1;
@@ -143,15 +193,13 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
       }
     }
     const float rstd = 1.0f / sqrtf(wave_sum(s2) / (float)a.K + a.eps);
-    const u32x4* g4 = reinterpret_cast<const u32x4*>(a.gamma);
-    const u32x4* b4 = reinterpret_cast<const u32x4*>(a.beta);
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = lane + i * 64;
       if (c < nchunk) {
-        const u32x4 g = g4[c], b = b4[c];
+        const in_t g = gw[i], b = bw[i];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < W; ++j) {
           const float y0 = f[i][2 * j] * rstd * bf16_lo_to_f32(g[j]) + bf16_lo_to_f32(b[j]);
           const float y1 = f[i][2 * j + 1] * rstd * bf16_hi_to_f32(g[j]) + bf16_hi_to_f32(b[j]);
           const unsigned int y = pack_bf16x2(y0, y1);  // the bf16 values a separate LayerNorm would have stored
@@ -166,8 +214,8 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
 #pragma unroll
   for (int i = 0; i < NCH; ++i)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(f[i][e]));
-  amax = wave_max(amax);
+    for (int e = 0; e < EPC; ++e) amax = fmaxf(amax, fabsf(f[i][e]));
+  amax = wave_max_nonneg(amax);
 
   const float scale = fmaxf(amax, 1e-5f) / 127.0f;
   const float inv_scale = 1.0f / scale;
@@ -176,29 +224,36 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = lane + i * 64;
-    if (c < nchunk) *dst_of(c) = quantize8(f[i], scale, inv_scale);
+    if (c < nchunk) {
+      unsigned int codes[EPC / 4];
+      quantize_chunk<EPC>(f[i], scale, inv_scale, codes);
+      store_chunk(c, codes);
+    }
   }
 }
 
-template <int NCH, bool LN>
+template <int NCH, int EPC, bool LN>
 static int launch_quant(const QuantArgs& a, hipStream_t stream) {
   const int64_t blocks = (a.M + kQuantWavesPerBlock - 1) / kQuantWavesPerBlock;
-  hipLaunchKernelGGL((quant_rowwise_bf16_kernel<NCH, LN>), dim3((unsigned int)blocks),
+  hipLaunchKernelGGL((quant_rowwise_bf16_kernel<NCH, EPC, LN>), dim3((unsigned int)blocks),
                      dim3(64 * kQuantWavesPerBlock), 0, stream, a);
   return check_launch("quant_rowwise_bf16_kernel");
 }
 
 template <bool LN>
 static int dispatch_quant(const QuantArgs& a, hipStream_t s) {
+  // rows that 4-element chunks divide among the 64 lanes exactly and 8-element chunks do not
+  if (a.K == 768) return launch_quant<3, 4, LN>(a, s);
+  if (a.K == 1280) return launch_quant<5, 4, LN>(a, s);
   const int need = (a.K / 8 + 63) / 64;
-  if (need <= 2) return launch_quant<2, LN>(a, s);
-  if (need <= 3) return launch_quant<3, LN>(a, s);
-  if (need <= 4) return launch_quant<4, LN>(a, s);
-  if (need <= 6) return launch_quant<6, LN>(a, s);
-  if (need <= 8) return launch_quant<8, LN>(a, s);
-  if (need <= 10) return launch_quant<10, LN>(a, s);
-  if (need <= 12) return launch_quant<12, LN>(a, s);
-  return launch_quant<16, LN>(a, s);
+  if (need <= 2) return launch_quant<2, 8, LN>(a, s);
+  if (need <= 3) return launch_quant<3, 8, LN>(a, s);
+  if (need <= 4) return launch_quant<4, 8, LN>(a, s);
+  if (need <= 6) return launch_quant<6, 8, LN>(a, s);
+  if (need <= 8) return launch_quant<8, 8, LN>(a, s);
+  if (need <= 10) return launch_quant<10, 8, LN>(a, s);
+  if (need <= 12) return launch_quant<12, 8, LN>(a, s);
+  return launch_quant<16, 8, LN>(a, s);
 }
 
 static int check_common(const char* who, const void* x, int64_t ldx, const int8_t* xq, const float* sx,
