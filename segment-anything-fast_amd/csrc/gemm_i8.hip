@@ -437,17 +437,20 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
     // tile), leaving tile kt+2 in flight across the barrier.
     constexpr int NLD = (GBM + GBN) / 64;  // wave instructions per tile and wave: 6 / 8
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    int dma_off[NLD];
+    // unsigned 32-bit lane offsets from a wave-uniform base: the loads then take the
+    // scalar-base form (global_load_lds_dwordx4 v_off, s[base]).  With 64-bit per-lane
+    // addresses each of them costs the MFMA stream ~100 cycles instead of ~15 (measured).
+    unsigned int dma_off[NLD];
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const int rho = 16 * (wave_u + 4 * i) + (lane >> 2);  // LDS row of this lane's chunk
       const int chunk = (lane & 3) ^ lds_swizzle(rho);
       if (i < GBM / 64) {  // X rows
-        dma_off[i] = min(m0 + rho, a.M - 1) * a.row_pitch + chunk * 16;
+        dma_off[i] = (unsigned int)(min(m0 + rho, a.M - 1) * a.row_pitch + chunk * 16);
       } else {             // W slots (slot s of a 128-column half holds W row (s%32)*4 + s/32)
         const int sl = rho - GBM;
         const int wrow = (sl & 128) + (sl & 31) * 4 + ((sl & 127) >> 5);
-        dma_off[i] = min(n0 + wrow, a.N - 1) * a.row_pitch + chunk * 16;
+        dma_off[i] = (unsigned int)(min(n0 + wrow, a.N - 1) * a.row_pitch + chunk * 16);
       }
     }
     typedef __attribute__((address_space(1))) const void* gptr_t;
@@ -455,9 +458,14 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
     auto dma_issue = [&](int kt, int stage_off) {
       const int8_t* xb = a.x + kt * a.x_kstep;
       const int8_t* wb = a.w + kt * a.w_kstep;
+      // keep the tile bases in scalar registers: folded into the lane offsets they would
+      // turn the loads back into the 64-bit per-lane address form
+      asm volatile("" : "+s"(xb), "+s"(wb));
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
-        const int8_t* src = (i < GBM / 64 ? xb : wb) + dma_off[i];
+        unsigned int off = dma_off[i];
+        asm volatile("" : "+v"(off));  // a 32-bit value at the point of use: no hoisted 64-bit copy
+        const int8_t* src = (i < GBM / 64 ? xb : wb) + off;
         unsigned char* dst = lds + stage_off + (wave_u + 4 * i) * 1024;
         __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
       }
