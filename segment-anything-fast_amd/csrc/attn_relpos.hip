@@ -156,24 +156,31 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
   typedef __attribute__((address_space(1))) const void* gptr_t;
   typedef __attribute__((address_space(3))) void* lptr_t;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  int koff[C::DPW], voff[C::DPW];
+  unsigned int koff[C::DPW], voff[C::DPW];  // unsigned lane offsets: scalar-base load form
+  bool dma_ok[C::DPW];
 #pragma unroll
   for (int m = 0; m < C::DPW; ++m) {
     const int P = 64 * (wave_u + 4 * m) + lane;
     const int row = P / C::PPR, col = P % C::PPR;
     const bool ok = (wave_u + 4 * m < C::NDMA) && col < HD / 8;
-    koff[m] = ok ? row * (int)a.k_sn + col * 8 : -1;
-    voff[m] = ok ? row * (int)a.v_sn + col * 8 : -1;
+    dma_ok[m] = ok;
+    koff[m] = ok ? (unsigned int)(row * (int)a.k_sn + col * 8) * 2u : 0u;  // bytes
+    voff[m] = ok ? (unsigned int)(row * (int)a.v_sn + col * 8) * 2u : 0u;
   }
   auto stage_dma = [&](int kt, int buf) {
-    const unsigned short* kb = kbase + (int64_t)kt * 64 * a.k_sn;
-    const unsigned short* vb = vbase + (int64_t)kt * 64 * a.v_sn;
+    const unsigned char* kb = reinterpret_cast<const unsigned char*>(kbase + (int64_t)kt * 64 * a.k_sn);
+    const unsigned char* vb = reinterpret_cast<const unsigned char*>(vbase + (int64_t)kt * 64 * a.v_sn);
+    // tile bases in scalar registers, 32-bit lane offsets at the point of use: the loads take the
+    // scalar-base form, which disturbs the MFMA stream several times less than 64-bit lane addresses
+    asm volatile("" : "+s"(kb), "+s"(vb));
     unsigned char* kl = lds + buf * C::STAGE + wave_u * 1024;
 #pragma unroll
     for (int m = 0; m < C::DPW; ++m) {
-      if (wave_u + 4 * m < C::NDMA && koff[m] >= 0) {
-        __builtin_amdgcn_global_load_lds((gptr_t)(kb + koff[m]), (lptr_t)(kl + m * 4096), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((gptr_t)(vb + voff[m]), (lptr_t)(kl + C::KBYTES + m * 4096), 16, 0, 0);
+      if (wave_u + 4 * m < C::NDMA && dma_ok[m]) {
+        unsigned int ok_ = koff[m], ov_ = voff[m];
+        asm volatile("" : "+v"(ok_), "+v"(ov_));
+        __builtin_amdgcn_global_load_lds((gptr_t)(kb + ok_), (lptr_t)(kl + m * 4096), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(vb + ov_), (lptr_t)(kl + C::KBYTES + m * 4096), 16, 0, 0);
       }
     }
   };

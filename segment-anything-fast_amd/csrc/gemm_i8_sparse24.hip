@@ -283,16 +283,16 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_kernel(SparseArgs a) {
   // ---- global -> LDS: per tile and wave 2 x (X, 16 B) + 2 x (Wc, 16 B) + 2 x (index, 4 B) ----
   constexpr int NLD = 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  int off_x[2], off_w[2], off_i[2];
+  unsigned int off_x[2], off_w[2], off_i[2];  // unsigned lane offsets: scalar-base load form
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int blk = wave_u + 4 * i;  // 1 KB block of the X / Wc tile, 256 B block of the index tile
     const int xr = 16 * blk + (lane >> 2);
-    off_x[i] = min(x0 + xr, a.M - 1) * a.x_row_pitch + (((lane & 3) ^ sp_swizzle_x(xr)) * 16);
+    off_x[i] = (unsigned int)(min(x0 + xr, a.M - 1) * a.x_row_pitch + (((lane & 3) ^ sp_swizzle_x(xr)) * 16));
     const int slot = 32 * blk + (lane >> 1);
     const int gn = min(w0 + sp_slot_to_row(slot), a.N - 1);
-    off_w[i] = gn * 32 + (((lane & 1) ^ sp_swizzle_w(slot)) * 16);
-    off_i[i] = gn * 8 + (lane & 1) * 4;
+    off_w[i] = (unsigned int)(gn * 32 + (((lane & 1) ^ sp_swizzle_w(slot)) * 16));
+    off_i[i] = (unsigned int)(gn * 8 + (lane & 1) * 4);
   }
   typedef __attribute__((address_space(1))) const void* gptr_t;
   typedef __attribute__((address_space(3))) void* lptr_t;
@@ -300,13 +300,19 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_kernel(SparseArgs a) {
     const int8_t* xb = a.x + kt * a.x_kstep;
     const int8_t* wb_ = a.wc + (int64_t)kt * a.N * 32;
     const int8_t* ib = reinterpret_cast<const int8_t*>(a.widx) + (int64_t)kt * a.N * 8;
+    // tile bases stay in scalar registers and the lane offsets 32-bit at the point of use, so the
+    // loads take the scalar-base form (the 64-bit per-lane address form costs the MFMA stream
+    // several times more per load)
+    asm volatile("" : "+s"(xb), "+s"(wb_), "+s"(ib));
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int blk = wave_u + 4 * i;
-      __builtin_amdgcn_global_load_lds((gptr_t)(xb + off_x[i]), (lptr_t)(lds + stage_off + blk * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_t)(wb_ + off_w[i]),
+      unsigned int ox = off_x[i], ow = off_w[i], oi = off_i[i];
+      asm volatile("" : "+v"(ox), "+v"(ow), "+v"(oi));
+      __builtin_amdgcn_global_load_lds((gptr_t)(xb + ox), (lptr_t)(lds + stage_off + blk * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(wb_ + ow),
                                        (lptr_t)(lds + stage_off + S_OFF_W + blk * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_t)(ib + off_i[i]),
+      __builtin_amdgcn_global_load_lds((gptr_t)(ib + oi),
                                        (lptr_t)(lds + stage_off + S_OFF_I + blk * 256), 4, 0, 0);
     }
   };
