@@ -1,9 +1,12 @@
 // Per-row symmetric int8 quantiser (bf16 -> int8 + fp32 scale), optionally preceded
-// by LayerNorm over the row and a row gather (window partition).  HBM-bound.
+// by LayerNorm over the row and a row gather (window partition).  HBM-bound for long rows
+// (K = 5120); for K = 1280, whose tensors sit in the last-level cache, the vector ALU is the
+// limit (about 360 instructions per row plain, 630 with LayerNorm).
 //
-// One wavefront owns one output row: the source row is read once with 16-byte loads
-// into registers, (normalised,) reduced to its absmax across the 64 lanes, then
-// scaled, rounded half-to-even and written back as 8-byte packs of int8.
+// One wavefront owns one output row: the source row is read once with 16- or 8-byte loads
+// and unpacked to fp32 registers, (normalised,) reduced to its absmax across the 64 lanes
+// (DPP within rows of 16 lanes, lane swaps between them: no LDS), then scaled, rounded
+// half-to-even and written back as 8- or 4-byte packs of int8.
 // Algorithmic traffic: 2 bytes read + 1 byte written per element + 4 bytes of scale.
 //
 // q = rint(x / s) must equal the IEEE division bit for bit.  Most elements take a
