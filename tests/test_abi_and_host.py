@@ -131,3 +131,41 @@ def test_composite_cpu_route_is_the_reference_fallback():
     got = _attention_rel_h_rel_w(q, k, v, rel_h, rel_w)
     assert torch.allclose(got, ora.attention_rel_h_rel_w(q, k, v, rel_h, rel_w), atol=1e-5)
     assert hasattr(torch.ops.customflash, "custom_flash_aligned")
+
+
+def test_checkpoint_with_reference_key_names_loads(tmp_path):
+    """A checkpoint in the layout the released SAM files have (key names follow the module
+    tree of the reference, modeling/image_encoder.py:15-120 and modeling/sam.py:18-58; prompt
+    encoder and mask decoder entries present) loads through the registry, and the quantised
+    modules are then built from the loaded weights."""
+    import samfast_amd
+    from samfast_amd import Int8DynamicLinear, apply_dynamic_quant
+    donor = samfast_amd.sam_model_registry["vit_b"]()
+    g = torch.Generator().manual_seed(11)
+    sd = {}
+    for k, v in donor.state_dict().items():
+        sd[k] = (torch.randn(v.shape, generator=g) * 0.02).to(torch.float16) if v.is_floating_point() else v
+    # what the module tree of the reference's encoder gives, written out by rule
+    expect = {"image_encoder.pos_embed", "image_encoder.patch_embed.proj.weight", "image_encoder.patch_embed.proj.bias",
+              "image_encoder.neck.0.weight", "image_encoder.neck.1.weight", "image_encoder.neck.1.bias",
+              "image_encoder.neck.2.weight", "image_encoder.neck.3.weight", "image_encoder.neck.3.bias"}
+    for i in range(12):
+        for leaf in ("norm1.weight", "norm1.bias", "attn.rel_pos_h", "attn.rel_pos_w", "attn.qkv.weight",
+                     "attn.qkv.bias", "attn.proj.weight", "attn.proj.bias", "norm2.weight", "norm2.bias",
+                     "mlp.lin1.weight", "mlp.lin1.bias", "mlp.lin2.weight", "mlp.lin2.bias"):
+            expect.add(f"image_encoder.blocks.{i}.{leaf}")
+    assert {k for k in sd if k.startswith("image_encoder.")} == expect
+    # entries of the parts that are not built here
+    sd["prompt_encoder.pe_layer.positional_encoding_gaussian_matrix"] = torch.zeros(2, 128)
+    sd["mask_decoder.iou_token.weight"] = torch.zeros(1, 256)
+    path = tmp_path / "sam_vit_b.pth"
+    torch.save(sd, path)
+    sam = samfast_amd.sam_model_registry["vit_b"](checkpoint=str(path))
+    w = sam.image_encoder.blocks[3].mlp.lin1.weight
+    assert torch.equal(w, sd["image_encoder.blocks.3.mlp.lin1.weight"].float())
+    assert sam.image_encoder.blocks[0].attn.rel_pos_h.shape == (27, 64)     # windowed block: 2*14-1
+    assert sam.image_encoder.blocks[2].attn.rel_pos_h.shape == (127, 64)    # global block: 2*64-1
+    apply_dynamic_quant(sam.image_encoder.blocks[3])
+    q = sam.image_encoder.blocks[3].mlp.lin1
+    assert isinstance(q, Int8DynamicLinear)
+    assert (q.weight - w).abs().max() <= q.sw.max() * 0.5001
