@@ -580,6 +580,18 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
 #pragma unroll
     for (int s = 0; s < C::KS; ++s) qf[s] = load_bf16x8_global(qp + 16 * s);
   }
+  // the table rows both bias products need (row min(lr, 2g-2) of rel_pos_h and of rel_pos_w):
+  // requested now, so that their latency runs under the K requests below
+  bf16x8 tfrag[FUSED ? 2 : 1][C::KS];
+  if (FUSED && has_tile) {
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+      const unsigned short* tab = which ? a.rw : a.rh;
+      const int trow = min(lr, 2 * (which ? a.gw : a.gh) - 2);
+#pragma unroll
+      for (int s = 0; s < C::KS; ++s) tfrag[which][s] = load_bf16x8_global(tab + trow * HD + 16 * s + 8 * lh);
+    }
+  }
   // wave instruction i of the window fills pieces 64i .. 64i+63: piece P is key P / PPR,
   // 16-byte column P % PPR (spare column and keys >= N: lane masked).  K goes first and travels
   // under the bias prologue; V follows once the scratch in its area is free.
@@ -621,17 +633,12 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
         // wave's scratch rows and read back at rel = qpos - slot + g - 1
         const int g = which ? a.gw : a.gh;
         const int qpos = which ? qw : qh;
-        const unsigned short* tab = which ? a.rw : a.rh;
-        const int trow = min(lr, 2 * g - 2);
         f32x16 tacc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) tacc[r] = 0.f;
         if (has_tile) {
-          bf16x8 tf[C::KS];
 #pragma unroll
-          for (int s = 0; s < C::KS; ++s) tf[s] = load_bf16x8_global(tab + trow * HD + 16 * s + 8 * lh);
-#pragma unroll
-          for (int s = 0; s < C::KS; ++s) tacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf[s], qf[s], tacc, 0, 0, 0);
+          for (int s = 0; s < C::KS; ++s) tacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tfrag[which][s], qf[s], tacc, 0, 0, 0);
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
