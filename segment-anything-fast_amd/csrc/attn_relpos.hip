@@ -607,13 +607,29 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     dma_col[m] = col * 8;
     dma_tok[m] = (row < N && col < HD / 8) ? tok_of(row) : -2;
   }
+  // Token rows and padding rows come from different allocations: one load per source, each with
+  // a wave-uniform base and an unsigned 32-bit lane offset (the scalar-base form disturbs the
+  // matrix pipe of the co-resident workgroup much less than 64-bit per-lane addresses); the two
+  // loads of an instruction slot have complementary lane masks and the same LDS block.
   auto window_dma = [&](const unsigned short* base, int64_t sn, const unsigned short* pad, unsigned char* dst) {
+    const unsigned char* tb = reinterpret_cast<const unsigned char*>(base);
+    const unsigned char* pb = reinterpret_cast<const unsigned char*>(pad);
+    asm volatile("" : "+s"(tb), "+s"(pb));
+    const unsigned int sn_bytes = (unsigned int)sn * 2u;
 #pragma unroll
     for (int m = 0; m < C::DPW; ++m) {
       const int inst = wave_u + C::WAVES * m;
-      if (64 * inst < N * C::PPR && dma_tok[m] > -2) {  // first test uniform
-        const unsigned short* src = (dma_tok[m] >= 0 ? base + (int64_t)dma_tok[m] * sn : pad) + dma_col[m];
-        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + inst * 1024), 16, 0, 0);
+      if (64 * inst < N * C::PPR) {  // uniform
+        if (dma_tok[m] >= 0) {
+          unsigned int off = (unsigned int)dma_tok[m] * sn_bytes + (unsigned int)dma_col[m] * 2u;
+          asm volatile("" : "+v"(off));
+          __builtin_amdgcn_global_load_lds((gptr_t)(tb + off), (lptr_t)(dst + inst * 1024), 16, 0, 0);
+        }
+        if (dma_tok[m] == -1) {
+          unsigned int off = (unsigned int)dma_col[m] * 2u;
+          asm volatile("" : "+v"(off));
+          __builtin_amdgcn_global_load_lds((gptr_t)(pb + off), (lptr_t)(dst + inst * 1024), 16, 0, 0);
+        }
       }
     }
   };
@@ -883,6 +899,11 @@ static int attn_dispatch(bool fused, AttnArgs& a, int hd, int dtype, float sm_sc
              "attn_relpos: q/k/v/out must be 16-byte aligned");
   SF_REQUIRE(a.q_sn >= hd && a.k_sn >= hd && a.v_sn >= hd && a.o_sn >= hd,
              "attn_relpos: token stride smaller than head_dim");
+  if (!global_path) {  // byte offsets of a token row inside its (batch, head) slice are kept in 32 bits
+    const int64_t toks = a.ws > 0 ? (int64_t)a.img_h * a.img_w : a.N;
+    SF_REQUIRE(toks * a.k_sn * 2 < (1ll << 32) && toks * a.v_sn * 2 < (1ll << 32),
+               "attn_relpos: k / v token stride too large for %lld tokens", (long long)toks);
+  }
   if (global_path)  // tile-relative element offsets are kept in 32 bits
     SF_REQUIRE(a.k_sn < (1 << 24) && a.v_sn < (1 << 24), "attn_relpos: k / v token stride too large");
   if (fused) {
