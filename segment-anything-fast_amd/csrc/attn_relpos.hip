@@ -657,9 +657,10 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
           for (int s = 0; s < C::KS; ++s) tacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tfrag[which][s], qf[s], tacc, 0, 0, 0);
         }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
+        for (int r = 0; r < 16; r += 2) {  // registers r, r+1 are adjacent rel: one packed 4-byte write
           const int rel = 8 * (r >> 2) + 4 * lh + (r & 3);
-          X[lr * C::XSTR + rel] = (unsigned short)f32_to_bf16_bits(tacc[r] * a.inv_scale);
+          *reinterpret_cast<unsigned int*>(X + lr * C::XSTR + rel) =
+              pack_bf16x2(tacc[r] * a.inv_scale, tacc[r + 1] * a.inv_scale);
         }
         wave_lds_fence();
 #pragma unroll
