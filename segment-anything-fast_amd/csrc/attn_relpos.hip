@@ -505,7 +505,7 @@ struct WindowCfg {
   // when HD is not a multiple of 32 the last output tile has spare rows: the spare piece of
   // every V row is preset to (1, 0, ..., 0) and row HD of O^T is the softmax denominator
   static constexpr bool ONES_ROW = HD % 32 != 0;
-  static constexpr int XSTR = 34;              // bf16 elements per scratch row
+  static constexpr int XSTR = 50;              // bf16 elements per scratch row: 32 products stored in reverse + read-ahead room; 25 words: odd, no bank conflicts
   static constexpr int XBYTES_WAVE = 32 * XSTR * 2;  // gather scratch, aliases the V area before V arrives
   static constexpr int LDS_BYTES = KBYTES + VBYTES;
   static_assert(WAVES * XBYTES_WAVE <= VBYTES, "gather scratch must fit in the V area");
@@ -657,23 +657,28 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
           for (int s = 0; s < C::KS; ++s) tacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tfrag[which][s], qf[s], tacc, 0, 0, 0);
         }
 #pragma unroll
+        // stored in reverse (position 31 - rel), so that the lane's eight slots 8lh .. 8lh+7, which
+        // want rel = qpos + g - 1 - slot, are eight consecutive positions E0 .. E0+7
         for (int r = 0; r < 16; r += 2) {  // registers r, r+1 are adjacent rel: one packed 4-byte write
           const int rel = 8 * (r >> 2) + 4 * lh + (r & 3);
-          *reinterpret_cast<unsigned int*>(X + lr * C::XSTR + rel) =
-              pack_bf16x2(tacc[r] * a.inv_scale, tacc[r + 1] * a.inv_scale);
+          *reinterpret_cast<unsigned int*>(X + lr * C::XSTR + 30 - rel) =
+              pack_bf16x2(tacc[r + 1] * a.inv_scale, tacc[r] * a.inv_scale);
         }
         wave_lds_fence();
+        {
+          const int e0 = 31 - (qpos + g - 1 - 8 * lh);  // 1 <= e0 <= 39 for 1 <= g <= 16
+          const unsigned int* xw = reinterpret_cast<const unsigned int*>(X + lr * C::XSTR) + (e0 >> 1);
+          unsigned int w[5];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          unsigned int pk2 = 0u;
+          for (int i = 0; i < 5; ++i) w[i] = xw[i];
+          const unsigned int sh = (e0 & 1) * 16;  // odd start: shift the pairs down by one element
 #pragma unroll
-          for (int v = 0; v < 2; ++v) {
-            const int slot = 8 * lh + 2 * i + v;
-            // unconditional read at a clamped position, then select
-            const unsigned int raw = X[lr * C::XSTR + max(0, min(qpos - slot + g - 1, 31))];
-            pk2 |= ((slot < g) ? raw : 0u) << (16 * v);
+          for (int i = 0; i < 4; ++i) {
+            const unsigned int pair = __builtin_amdgcn_alignbit(w[i + 1], w[i], sh);
+            const int slot = 8 * lh + 2 * i;  // positions past the table (slot >= g) hold no product: zero
+            const unsigned int mask = (slot < g ? 0xffffu : 0u) | (slot + 1 < g ? 0xffff0000u : 0u);
+            if (which) bww[i] = pair & mask; else bhw[i] = pair & mask;
           }
-          if (which) bww[i] = pk2; else bhw[i] = pk2;
         }
         wave_lds_fence();
       }
