@@ -96,13 +96,15 @@ SF_DEVICE float max_with_lane_xor32(float v) {
 SF_DEVICE void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 // =============================================================================
-// global kernel: gw == 64, N % (128*QT) == 0
+// global kernel: gw == 64, N % (32*WAVES*QT) == 0.  WAVES = 4: two workgroups per CU; WAVES = 8:
+// one workgroup of 256 queries per CU, which stages every K / V tile once for twice the queries
+// (the global->LDS loads are a fifth of the kernel's time), taken when the grid is large enough
 // =============================================================================
-template <int HD, int QT>
+template <int HD, int QT, int WAVES>
 struct GlobalCfg {
   static constexpr int KS = HD / 16;          // score k-steps
   static constexpr int DT = (HD + 31) / 32;   // output channel tiles
-  static constexpr int BM = 128 * QT;         // queries per workgroup
+  static constexpr int BM = 32 * WAVES * QT;  // queries per workgroup
   // K and V tiles travel global memory -> LDS directly (global_load_lds_dwordx4), row-major,
   // in 16-byte pieces: a staged row is HD/8 data pieces plus one spare piece that no load
   // writes (its lanes are masked), so rows are HD + 8 elements apart (bank spread) and 64 rows
@@ -121,15 +123,16 @@ struct GlobalCfg {
   static constexpr int RELH_BYTES = 64 * BM * 4;
   static constexpr int LDS_BYTES = RELH_OFF + RELH_BYTES;
   static constexpr int XSTR = 65;             // gather scratch row stride (floats)
-  static constexpr int X_BYTES = 4 * 32 * XSTR * 4;
+  static constexpr int X_BYTES = WAVES * 32 * XSTR * 4;
   static constexpr int NDMA = PPR;            // wave instructions per K (or V) tile
-  static constexpr int DPW = (NDMA + 3) / 4;  // of which each of the 4 waves issues at most
-  static_assert(X_BYTES <= 2 * STAGE, "gather scratch must fit in the K/V stages");
+  static constexpr int DPW = (NDMA + WAVES - 1) / WAVES;  // of which each wave issues at most
+  // the scratch is dead (barrier) before the stages and relhT are written
+  static_assert(X_BYTES <= LDS_BYTES, "gather scratch must fit in the workgroup's LDS");
 };
 
-template <int HD, int QT, bool FUSED>
-__global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
-  using C = GlobalCfg<HD, QT>;
+template <int HD, int QT, bool FUSED, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_kernel(AttnArgs a) {
+  using C = GlobalCfg<HD, QT, WAVES>;
   __shared__ __attribute__((aligned(16))) unsigned char lds[C::LDS_BYTES];
   float* relhT = reinterpret_cast<float*>(lds + C::RELH_OFF);  // [kh][BM]
 
@@ -160,9 +163,9 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
   bool dma_ok[C::DPW];
 #pragma unroll
   for (int m = 0; m < C::DPW; ++m) {
-    const int P = 64 * (wave_u + 4 * m) + lane;
+    const int P = 64 * (wave_u + WAVES * m) + lane;
     const int row = P / C::PPR, col = P % C::PPR;
-    const bool ok = (wave_u + 4 * m < C::NDMA) && col < HD / 8;
+    const bool ok = (wave_u + WAVES * m < C::NDMA) && col < HD / 8;
     dma_ok[m] = ok;
     koff[m] = ok ? (unsigned int)(row * (int)a.k_sn + col * 8) * 2u : 0u;  // bytes
     voff[m] = ok ? (unsigned int)(row * (int)a.v_sn + col * 8) * 2u : 0u;
@@ -176,11 +179,11 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
     unsigned char* kl = lds + buf * C::STAGE + wave_u * 1024;
 #pragma unroll
     for (int m = 0; m < C::DPW; ++m) {
-      if (wave_u + 4 * m < C::NDMA && dma_ok[m]) {
+      if (wave_u + WAVES * m < C::NDMA && dma_ok[m]) {
         unsigned int ok_ = koff[m], ov_ = voff[m];
         asm volatile("" : "+v"(ok_), "+v"(ov_));
-        __builtin_amdgcn_global_load_lds((gptr_t)(kb + ok_), (lptr_t)(kl + m * 4096), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((gptr_t)(vb + ov_), (lptr_t)(kl + C::KBYTES + m * 4096), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(kb + ok_), (lptr_t)(kl + m * WAVES * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(vb + ov_), (lptr_t)(kl + C::KBYTES + m * WAVES * 1024), 16, 0, 0);
       }
     }
   };
@@ -316,7 +319,7 @@ __global__ __launch_bounds__(256, 2) void attn_global_kernel(AttnArgs a) {
   } else {
     first_tile();
     const unsigned short* rhb = a.rh + b * a.rh_sb + h * a.rh_sh + (int64_t)q_wg * a.rh_sn;
-    for (int idx = tid; idx < C::BM * a.gh; idx += 256) {
+    for (int idx = tid; idx < C::BM * a.gh; idx += 64 * WAVES) {
       const int ql = idx % C::BM, kh = idx / C::BM;
       relhT[kh * C::BM + ql] = bf16_bits_to_f32(rhb[(int64_t)ql * a.rh_sn + kh]) * kLog2e;
     }
@@ -859,10 +862,20 @@ template <int HD, bool FUSED>
 static int launch_hd(const AttnArgs& a, bool global_path, hipStream_t stream) {
   if (global_path) {
     constexpr int QT = 1;
-    using C = GlobalCfg<HD, QT>;
-    const int64_t total = (int64_t)a.B * a.nH * (a.N / C::BM);
-    const unsigned int grid = (unsigned int)(((total + 7) / 8) * 8);
-    hipLaunchKernelGGL((attn_global_kernel<HD, QT, FUSED>), dim3(grid), dim3(256), 0, stream, a);
+    auto launch = [&](auto wc) {
+      constexpr int WAVES = decltype(wc)::value;
+      using C = GlobalCfg<HD, QT, WAVES>;
+      const int64_t total = (int64_t)a.B * a.nH * (a.N / C::BM);
+      const unsigned int grid = (unsigned int)(((total + 7) / 8) * 8);
+      hipLaunchKernelGGL((attn_global_kernel<HD, QT, FUSED, WAVES>), dim3(grid), dim3(64 * WAVES), 0, stream, a);
+    };
+    // 256 queries per workgroup when that still gives every CU several workgroups
+    // (SAMFAST_ATTN_WAVES=4 / 8 overrides the choice where the shape allows it)
+    const int64_t wg8 = (int64_t)a.B * a.nH * (a.N / 256);
+    const char* force = getenv("SAMFAST_ATTN_WAVES");
+    const bool want8 = force ? atoi(force) == 8 : wg8 >= 1024;
+    if (a.N % 256 == 0 && want8) launch(std::integral_constant<int, 8>{});
+    else launch(std::integral_constant<int, 4>{});
     return check_launch("attn_global_kernel");
   }
   const int64_t wins = a.ws > 0 ? (int64_t)a.B * a.wins_x * a.wins_y : a.B;

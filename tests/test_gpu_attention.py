@@ -202,3 +202,19 @@ def test_rising_maximum_along_the_keys(gh, gw, hd, ramp):
     out = ops.attn_relpos(q.to(dev), k.to(dev), v.to(dev), rph.to(dev), rpw.to(dev), (gh, gw))
     torch.cuda.synchronize()
     _check(out, ref, f"rising max {gh}x{gw}x{hd} ramp {ramp}")
+
+
+def test_global_kernel_wave_count_variants_agree(monkeypatch):
+    """The global kernel runs with 128 or 256 queries per workgroup (4 or 8 wavefronts); the choice
+    follows the grid size and can be forced.  A query's arithmetic does not depend on it."""
+    from samfast_amd import ops
+    B, nH, gh, gw, hd = 1, 2, 64, 64, 80
+    q, k, v, rph, rpw = (t.cuda() for t in attn_inputs(B, nH, gh, gw, hd, seed=5))
+    outs = {}
+    for waves in ("4", "8"):
+        monkeypatch.setenv("SAMFAST_ATTN_WAVES", waves)
+        outs[waves] = ops.attn_relpos(q, k, v, rph, rpw, (gh, gw)).clone()
+    torch.cuda.synchronize()
+    assert torch.equal(outs["4"], outs["8"])
+    ref = _oracle_tables(q.cpu(), k.cpu(), v.cpu(), rph.cpu(), rpw.cpu(), (gh, gw))
+    _check(outs["8"], ref, "8 wavefronts per workgroup")
