@@ -152,7 +152,8 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
     const int c = lane + i * 64;
     const in_t z = {};
     xw[i] = z;
-    if (c < nchunk) xw[i] = src[c];
+    // long rows (the 671 MB lin1 output at ViT-H batch 16) are read once and never again: streamed
+    if (c < nchunk) xw[i] = (!LN && NCH >= 8) ? __builtin_nontemporal_load(src + c) : src[c];
   }
   if (LN) {
     const in_t* g4 = reinterpret_cast<const in_t*>(a.gamma);
