@@ -271,7 +271,8 @@ SF_DEVICE void gemm_epilogue_staged(const GemmArgs& a, i32x16 (&acc)[2][4], unsi
 #pragma unroll
     for (int p = 0; p < 16; ++p) {
       if (EPI == EPI_RESIDUAL_BF16) add_residual(val[p], res[p]);
-      *reinterpret_cast<u32x4*>(op + (int64_t)(8 * p) * a.ldo) = val[p];
+      if (EPI == EPI_GELU_BF16 || EPI == EPI_SCALE_BIAS_BF16) __builtin_nontemporal_store(val[p], reinterpret_cast<u32x4*>(op + (int64_t)(8 * p) * a.ldo));
+      else *reinterpret_cast<u32x4*>(op + (int64_t)(8 * p) * a.ldo) = val[p];
     }
   } else {
 #pragma unroll
