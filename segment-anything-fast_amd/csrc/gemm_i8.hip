@@ -55,6 +55,7 @@ struct GemmArgs {
   int64_t ldo;
   int M, N, K;
   int tiles_m, tiles_n;
+  int stream_out;  // outputs without residual that exceed the 256 MB last-level cache
   int row_pitch;            // bytes between consecutive rows of X / W: K (row-major) or 64 (K-block major)
   int64_t x_kstep, w_kstep; // bytes between consecutive 64-byte k tiles: 64, or rows * 64
   const unsigned short* residual;  // EPI_RESIDUAL: (rows, N) bf16, row stride ld_res
@@ -271,7 +272,8 @@ SF_DEVICE void gemm_epilogue_staged(const GemmArgs& a, i32x16 (&acc)[2][4], unsi
 #pragma unroll
     for (int p = 0; p < 16; ++p) {
       if (EPI == EPI_RESIDUAL_BF16) add_residual(val[p], res[p]);
-      if (EPI == EPI_GELU_BF16 || EPI == EPI_SCALE_BIAS_BF16) __builtin_nontemporal_store(val[p], reinterpret_cast<u32x4*>(op + (int64_t)(8 * p) * a.ldo));
+      // an output larger than the last-level cache that is read once (qkv, lin1) is streamed out
+      if (a.stream_out) __builtin_nontemporal_store(val[p], reinterpret_cast<u32x4*>(op + (int64_t)(8 * p) * a.ldo));
       else *reinterpret_cast<u32x4*>(op + (int64_t)(8 * p) * a.ldo) = val[p];
     }
   } else {
@@ -606,6 +608,7 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   const int bm = 64 * tm;
   a.tiles_m = (int)((M + bm - 1) / bm);
   a.tiles_n = (N + GBN - 1) / GBN;
+  a.stream_out = (epi == EPI_SCALE_BIAS_BF16 || epi == EPI_GELU_BF16) && M * (int64_t)N * 2 >= (256ll << 20);
   const int64_t total = (int64_t)a.tiles_m * a.tiles_n;
   SF_REQUIRE(total < (1ll << 30), "gemm_i8: too many tiles");
   const unsigned int grid = (unsigned int)(((total + 7) / 8) * 8);
