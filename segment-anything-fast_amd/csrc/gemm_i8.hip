@@ -55,6 +55,7 @@ struct GemmArgs {
   int64_t ldo;
   int M, N, K;
   int tiles_m, tiles_n;
+  int group_m;     // row tiles per scheduling group
   int stream_out;  // outputs without residual that exceed the 256 MB last-level cache
   int row_pitch;            // bytes between consecutive rows of X / W: K (row-major) or 64 (K-block major)
   int64_t x_kstep, w_kstep; // bytes between consecutive 64-byte k tiles: 64, or rows * 64
@@ -311,7 +312,7 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
   const unsigned int total = (unsigned int)a.tiles_m * (unsigned int)a.tiles_n;
   const unsigned int pid = xcd_contiguous_id(blockIdx.x, total);
   if (pid >= total) return;  // uniform over the workgroup
-  constexpr int GGROUP_M = 16 / TM;  // 1024 output rows per group: their X panels (1.3 MB at K=1280) stay in L2
+  const unsigned int GGROUP_M = a.group_m;
   const unsigned int per_group = GGROUP_M * a.tiles_n;
   const unsigned int first_m = (pid / per_group) * GGROUP_M;
   const unsigned int gsz = min((unsigned int)a.tiles_m - first_m, (unsigned int)GGROUP_M);
@@ -608,6 +609,10 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   const int bm = 64 * tm;
   a.tiles_m = (int)((M + bm - 1) / bm);
   a.tiles_n = (N + GBN - 1) / GBN;
+  // row tiles per scheduling group, from the fabric traffic measured per shape: with few column
+  // tiles (proj, lin2: 5) the workgroups that share an X row tile should be adjacent (-23 % / -31 %
+  // fetched bytes); with many (qkv 15, lin1 20) 1024 rows per group let W panels be shared
+  a.group_m = a.tiles_n <= 6 ? 1 : 1024 / bm;
   a.stream_out = (epi == EPI_SCALE_BIAS_BF16 || epi == EPI_GELU_BF16) && M * (int64_t)N * 2 >= (256ll << 20);
   const int64_t total = (int64_t)a.tiles_m * a.tiles_n;
   SF_REQUIRE(total < (1ll << 30), "gemm_i8: too many tiles");
