@@ -27,9 +27,17 @@
 // after the K loop every lane owns 4 adjacent columns of each of its rows and writes
 // them with one 8-byte (bf16) or 16-byte (int32) store.
 //
-// Workgroup ids are first made contiguous per XCD, then walked in groups of 1024 output
-// rows x all column tiles so that the tiles resident on one XCD share their X panels
-// and the W matrix in that XCD's L2.
+// The loads use a wave-uniform base and an unsigned 32-bit lane offset
+// (global_load_lds_dwordx4 v_off, s[base:base+1]): each costs the MFMA stream ~15 cycles,
+// against ~100 with a 64-bit address per lane, which is the form the compiler picks unless
+// the base is pinned in scalar registers and the offset kept 32-bit at the point of use.
+//
+// Workgroup ids are first made contiguous per XCD, then walked in groups of row tiles x all
+// column tiles so that the tiles resident on one XCD share operand panels in that XCD's L2:
+// 1024 rows per group when there are many column tiles (W panels shared), one row tile per
+// group when there are few (the column tiles of a row tile run side by side and share X).
+// Outputs larger than the last-level cache that carry no residual (qkv, lin1: read once by
+// the next kernel) are written with streaming stores.
 #include "samfast_internal.hpp"
 #include <stdlib.h>
 #include <type_traits>
