@@ -204,11 +204,12 @@ def test_rising_maximum_along_the_keys(gh, gw, hd, ramp):
     _check(out, ref, f"rising max {gh}x{gw}x{hd} ramp {ramp}")
 
 
-def test_global_kernel_wave_count_variants_agree(monkeypatch):
+@pytest.mark.parametrize("hd,gh", [(80, 64), (64, 64), (80, 8)])
+def test_global_kernel_wave_count_variants_agree(monkeypatch, hd, gh):
     """The global kernel runs with 128 or 256 queries per workgroup (4 or 8 wavefronts); the choice
     follows the grid size and can be forced.  A query's arithmetic does not depend on it."""
     from samfast_amd import ops
-    B, nH, gh, gw, hd = 1, 2, 64, 64, 80
+    B, nH, gw = 1, 2, 64
     q, k, v, rph, rpw = (t.cuda() for t in attn_inputs(B, nH, gh, gw, hd, seed=5))
     outs = {}
     for waves in ("4", "8"):
