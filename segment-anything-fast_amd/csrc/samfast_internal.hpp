@@ -62,22 +62,25 @@ SF_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 // value held by lane (lane ^ 32) of the same wavefront
 SF_DEVICE float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
-// GELU(x) = x * Phi(x) with 1 - Phi(|x|) = 0.5 * erfc(|x| / sqrt 2) from the
-// Abramowitz-Stegun 7.1.26 polynomial (|error| < 1.5e-7), written so that the negative
-// side keeps its relative accuracy:  gelu(x) = max(x, 0) - |x| * h,
-//   h = 0.5 * poly(t) * exp(-x^2 / 2),  t = 1 / (1 + p |x| / sqrt 2).
+// GELU(x) = x * Phi(x), written so that the negative side keeps its relative accuracy:
+//   gelu(x) = max(x, 0) - |x| * h,   h = Phi(-|x|) = 2^P(|x|),
+// P = degree-7 least-squares fit (Chebyshev nodes) of log2 Phi(-z) on [0, 6]: |P - log2 Phi|
+// < 7e-6, i.e. h to 5e-6 relative in fp32 Horner form - a result that differs from the
+// correctly rounded bf16 value in about one of a thousand cases, by one step.  Beyond |x| = 6
+// h is held at Phi(-6) = 1e-9.  One transcendental and ten other instructions per value.
 SF_DEVICE float gelu_erf(float x) {
 #pragma clang fp contract(fast)  // an approximation anyway: let the polynomial use FMAs
   const float ax = fabsf(x);
-  const float t = __builtin_amdgcn_rcpf(fmaf(ax, 0.3275911f * 0.70710678118654752f, 1.0f));
-  const float w = ax * 0.84932180028801904f;  // sqrt(log2(e) / 2): exp(-x^2/2) = exp2(-w^2)
-  const float e = __builtin_amdgcn_exp2f(-(w * w));
-  float poly = 0.5f * 1.061405429f;            // the 0.5 of h is folded into the coefficients
-  poly = fmaf(poly, t, 0.5f * -1.453152027f);
-  poly = fmaf(poly, t, 0.5f * 1.421413741f);
-  poly = fmaf(poly, t, 0.5f * -0.284496736f);
-  poly = fmaf(poly, t, 0.5f * 0.254829592f);
-  const float h = poly * t * e;
+  const float z = fminf(ax, 6.0f);
+  float p = -1.88962623e-06f;
+  p = fmaf(p, z, 6.26814010e-05f);
+  p = fmaf(p, z, -9.38867933e-04f);
+  p = fmaf(p, z, 8.53946133e-03f);
+  p = fmaf(p, z, -5.40206871e-02f);
+  p = fmaf(p, z, -4.58409777e-01f);
+  p = fmaf(p, z, -1.15126915e+00f);
+  p = fmaf(p, z, -9.99994340e-01f);
+  const float h = __builtin_amdgcn_exp2f(p);
   return fmaf(-ax, h, fmaxf(x, 0.f));
 }
 
