@@ -35,6 +35,7 @@ struct QuantArgs {
   int64_t M;
   int K;
   float eps;
+  float inv_K;  // 1 / K for the LayerNorm statistics
   int kb64;  // 1: write xq K-block major, (K/64, M, 64)
 };
 
@@ -182,7 +183,9 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
     for (int i = 0; i < NCH; ++i)
 #pragma unroll
       for (int j = 0; j < W; ++j) s1 += f[i][2 * j] + f[i][2 * j + 1];
-    const float mean = wave_sum(s1) / (float)a.K;
+    // statistics: multiplication by 1/K and a hardware reciprocal square root (1 ulp each; the
+    // LayerNorm result is compared with the reference to one code step, not bit for bit)
+    const float mean = wave_sum(s1) * a.inv_K;
     float s2 = 0.f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
@@ -196,7 +199,7 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
         }
       }
     }
-    const float rstd = 1.0f / sqrtf(wave_sum(s2) / (float)a.K + a.eps);
+    const float rstd = __builtin_amdgcn_rsqf(fmaf(wave_sum(s2), a.inv_K, a.eps));
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = lane + i * 64;
@@ -307,7 +310,7 @@ extern "C" int samfast_layernorm_quant_i8(const void* x, int64_t ldx, const void
   a.ldx = ldx; a.xq = xq; a.sx = sx; a.M = M; a.K = K;
   a.gamma = reinterpret_cast<const unsigned short*>(gamma);
   a.beta = reinterpret_cast<const unsigned short*>(beta);
-  a.src_row = src_row; a.eps = eps;
+  a.src_row = src_row; a.eps = eps; a.inv_K = 1.0f / (float)K;
   a.kb64 = layout == SAMFAST_LAYOUT_KB64;
   return dispatch_quant<true>(a, reinterpret_cast<hipStream_t>(stream));
 }
