@@ -219,3 +219,29 @@ def test_global_kernel_wave_count_variants_agree(monkeypatch, hd, gh):
     assert torch.equal(outs["4"], outs["8"])
     ref = _oracle_tables(q.cpu(), k.cpu(), v.cpu(), rph.cpu(), rpw.cpu(), (gh, gw))
     _check(outs["8"], ref, "8 wavefronts per workgroup")
+
+
+@pytest.mark.parametrize("batch", [1, 8])
+@pytest.mark.parametrize("head,hidden_dim", [(16, 80), (12, 64)])
+def test_reference_test_recipe_against_sdpa(batch, head, hidden_dim):
+    """The reference's own test of this operator (test/test_flash_4.py:5-43): its shapes (batch 1
+    and 8, 16 heads x 80 / 12 heads x 64, 4096 tokens), its input recipe (seed 20, q / k / v and
+    both bias factors ~ N(0, 0.5)) and its tolerance (rtol = atol = 1e-3) against
+    scaled_dot_product_attention with the materialised bias, here for the dtype the kernels are
+    built for (bf16); SDPA is evaluated in fp32 on the same bf16 inputs and rounded once."""
+    from samfast_amd.flash_4 import _attention_rel_h_rel_w
+    seq_len, dtype, device = 4096, torch.bfloat16, "cuda"
+    print(f"case reference recipe batch={batch} head={head} hd={hidden_dim}", flush=True)
+    torch.manual_seed(20)
+    q, k, v = (torch.empty((batch, head, seq_len, hidden_dim), dtype=dtype, device=device).normal_(mean=0.0, std=0.5)
+               for _ in range(3))
+    w = int(seq_len ** 0.5)
+    rel_h = torch.empty((batch, head, seq_len, w, 1), dtype=dtype, device=device).normal_(mean=0, std=0.5)
+    rel_w = torch.empty((batch, head, seq_len, 1, w), dtype=dtype, device=device).normal_(mean=0, std=0.5)
+    out = _attention_rel_h_rel_w(q, k, v, rel_h, rel_w)
+    assert out.dtype == dtype and out.shape == q.shape
+    for b in range(batch):  # one image at a time: the bias is 1 GB per image in fp32
+        bias = (rel_h[b:b + 1].float() + rel_w[b:b + 1].float()).view(1, head, seq_len, seq_len)
+        ref = torch.nn.functional.scaled_dot_product_attention(
+            q[b:b + 1].float(), k[b:b + 1].float(), v[b:b + 1].float(), attn_mask=bias)
+        torch.testing.assert_close(ref.to(dtype), out[b:b + 1], rtol=1e-3, atol=1e-3)
