@@ -90,6 +90,43 @@ def test_full_size_checksum():
     assert np.array_equal(acc[rows.cuda()].cpu().numpy().astype(np.int64), sub)
 
 
+@pytest.mark.parametrize("name,N,K", [("qkv", 3840, 1280), ("proj", 1280, 1280), ("lin1", 5120, 1280),
+                                      ("lin2", 1280, 5120)])
+def test_vit_h_linear_shapes_with_outlier_rows(name, N, K):
+    """The four ViT-H linears at M = 16 * 4096 tokens with the stated recipe: bf16 activations
+    ~ N(0, 1) with 0.1 % of the rows scaled 20x, weights ~ N(0, 0.02) quantised per output channel
+    (absmax / 127), activations per token the same way, seed 4.  Bit-exact: every activation code
+    and scale (the whole matrix against the oracle), the int32 accumulators (column sums of the
+    whole matrix against an exact int64 product, all outlier rows and a random row subset element
+    by element) and the bf16 outputs of the fused scale-and-bias epilogue on those rows."""
+    from samfast_amd import ops
+    from samfast_amd.quant import quantize_weight_per_channel
+    M = 16 * 4096
+    print(f"case vit_h linear {name} M={M} N={N} K={K}", flush=True)
+    x, w, b = linear_inputs(M, K, N, seed=4)
+    xq_ref, sx_ref = orq.quantize_rows_absmax(x)
+    xq, sx = ops.quant_rowwise(x.cuda())
+    assert np.array_equal(sx.cpu().numpy(), sx_ref)
+    assert np.array_equal(xq.cpu().numpy(), xq_ref)
+    wq, sw = quantize_weight_per_channel(w.float())
+    wq_ref, sw_ref = orq.quantize_rows_absmax(w.float())
+    assert np.array_equal(wq.numpy(), wq_ref) and np.array_equal(sw.numpy(), sw_ref)
+    acc = ops.gemm_i8_i32(xq, wq.cuda())
+    col_sum = acc.to(torch.int64).sum(dim=0).cpu().numpy()
+    expect = xq_ref.sum(axis=0, dtype=np.int64) @ wq_ref.astype(np.int64).T
+    assert np.array_equal(col_sum, expect)
+    g = torch.Generator().manual_seed(44)
+    outliers = torch.nonzero(x.float().abs().amax(dim=1) > 30.0).flatten()  # the 20x rows
+    assert 40 <= outliers.numel() <= 70
+    rows = torch.cat([outliers, torch.randperm(M, generator=g)[:64]])
+    sub = orq.int8_gemm_i64(xq_ref[rows.numpy()], wq_ref)
+    assert np.array_equal(acc[rows.cuda()].cpu().numpy().astype(np.int64), sub)
+    bias = b.float()
+    y = ops.gemm_i8_scale_bias(xq, sx, wq.cuda(), sw.cuda(), bias.cuda())
+    y_ref = orq.scale_bias_epilogue(sub.astype(np.int32), sx_ref[rows.numpy()], sw_ref, bias.numpy())
+    assert torch.equal(y[rows.cuda()].cpu().view(torch.int16), y_ref.view(torch.int16))
+
+
 def test_module_swap_forward():
     """apply_dynamic_quant swaps Linears; forward equals the oracle's dynamic linear."""
     from samfast_amd import apply_dynamic_quant
