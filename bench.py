@@ -56,6 +56,10 @@ def parse():
     p.add_argument("--calibration-copy", action="store_true",
                    help="also run one 1 GiB device-to-device copy (a known-size reference for "
                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
+    p.add_argument("--library-yardsticks", action="store_true",
+                   help="also time the ROCm libraries on the encoder's operator shapes (torch._int_mm = "
+                        "hipBLASLt int8, bf16 F.linear, F.scaled_dot_product_attention) next to the "
+                        "hand-written kernels; adds a 'library_yardsticks' object to the JSON line")
     return p.parse_args()
 
 
@@ -85,6 +89,70 @@ def kernel_table(summary):
             "unit": unit, "frac": round(rate / peak, 4),
         }
     return rows
+
+
+def library_yardsticks(batch, heads, hd, width):
+    """The encoder's operator shapes on the ROCm libraries that PyTorch calls, next to the kernels of
+    this repository on the same operands (events around 10 calls each, after 2 warm-up calls)."""
+    import torch
+    import torch.nn.functional as F
+    from samfast_amd import _lib, ops
+
+    def rate(fn, work, n=10):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return round(work / (e0.elapsed_time(e1) / n * 1e-3) / 1e12, 1)
+
+    res = {"unit": "TOP/s (linears), TFLOP/s (attention)", "linears": {}, "attention": {}}
+    M = batch * 4096
+    g = torch.Generator(device="cuda").manual_seed(4)
+    epi = {"qkv": _lib.EPILOGUE_NONE, "proj": _lib.EPILOGUE_RESIDUAL, "lin1": _lib.EPILOGUE_GELU,
+           "lin2": _lib.EPILOGUE_RESIDUAL}
+    for name, N, K in (("qkv", 3 * width, width), ("proj", width, width), ("lin1", 4 * width, width),
+                       ("lin2", width, 4 * width)):
+        x = torch.randn((M, K), device="cuda", generator=g)
+        x[torch.randperm(M, device="cuda", generator=g)[:max(1, M // 1000)]] *= 20.0
+        x = x.to(torch.bfloat16)
+        w = (torch.randn((N, K), device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+        xq, sx = ops.quant_rowwise(x)
+        wq, sw = ops.quant_rowwise(w)
+        xk, wk = ops.to_kb64(xq), ops.to_kb64(wq)
+        bias = torch.zeros(N, device="cuda")
+        resid = torch.randn((M, N), device="cuda").to(torch.bfloat16) if epi[name] == _lib.EPILOGUE_RESIDUAL else None
+        out = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        work = 2.0 * M * N * K
+        row = {"this_repo_fused_epilogue_bf16_out": rate(
+            lambda: ops.gemm_i8_fused(xk, sx, wk, sw, bias, epi[name], residual=resid, out=out,
+                                      layout=_lib.LAYOUT_KB64), work)}
+        try:
+            wt = wq.t()
+            row["torch_int_mm_int32_out"] = rate(lambda: torch._int_mm(xq, wt), work)
+        except Exception as e:  # not every build exposes it
+            row["torch_int_mm_int32_out"] = f"unavailable: {str(e)[:60]}"
+        row["torch_bf16_linear"] = rate(lambda: F.linear(x, w), work)
+        res["linears"][name] = row
+        del x, w, xq, wq, xk, wk, out, resid
+    for what, B, N, grid in (("global", batch, 4096, (64, 64)), ("window", batch * 25, 196, (14, 14))):
+        q, k, v = (torch.randn((B, heads, N, hd), device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+        rph = (torch.randn((2 * grid[0] - 1, hd), device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+        rpw = (torch.randn((2 * grid[1] - 1, hd), device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+        work = 4.0 * B * heads * N * N * hd
+        row = {"this_repo_with_relpos_bias": rate(lambda: ops.attn_relpos(q, k, v, rph, rpw, grid, hd ** -0.5), work),
+               "torch_sdpa_no_bias": rate(lambda: F.scaled_dot_product_attention(q, k, v), work)}
+        bias = torch.randn((B, heads, N, N), device="cuda", generator=g).to(torch.bfloat16)
+        row["torch_sdpa_materialised_bias"] = rate(
+            lambda: F.scaled_dot_product_attention(q, k, v, attn_mask=bias), work, n=3)
+        res["attention"][what] = row
+        del q, k, v, bias
+    torch.cuda.empty_cache()
+    return res
 
 
 def main():
@@ -204,6 +272,12 @@ def main():
                                   "min_cosine_vs_this_path": round(cos, 6)}
         del base, ref
         torch.cuda.empty_cache()
+
+    if args.library_yardsticks:
+        blk = enc.blocks[0].attn
+        with torch.no_grad():
+            result["library_yardsticks"] = library_yardsticks(
+                args.batch, blk.num_heads, blk.qkv.in_features // blk.num_heads, blk.qkv.in_features)
 
     if not args.no_cpu_baseline:
         from oracle import image_encoder as oe
