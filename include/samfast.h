@@ -14,7 +14,10 @@
  *   - strides are in ELEMENTS; the innermost (head_dim / K) axis is contiguous
  *     and every row start must be 16-byte aligned;
  *   - return value 0 = ok; negative = SAMFAST_E_*; the text of the last error
- *     on the calling thread is returned by samfast_last_error().
+ *     on the calling thread is returned by samfast_last_error();
+ *   - a call with no rows (M == 0) or no images (B == 0) is valid: the shape is
+ *     checked, nothing is launched, 0 is returned, and the buffers that would
+ *     hold those rows may be NULL (an empty tensor's data pointer).
  *
  * The reference interfaces each entry point stands in for are cited as
  * file:line under segment_anything_fast/ of pytorch-labs/segment-anything-fast.

@@ -886,9 +886,10 @@ static int launch_hd(const AttnArgs& a, bool global_path, hipStream_t stream) {
 
 static int attn_dispatch(bool fused, AttnArgs& a, int hd, int dtype, float sm_scale,
                          hipStream_t stream) {
-  SF_REQUIRE(a.q && a.k && a.v && a.out && a.rh && a.rw, "attn_relpos: null pointer");
-  SF_REQUIRE(a.B > 0 && a.nH > 0 && a.gh > 0 && a.gw > 0, "attn_relpos: bad shape");
+  SF_REQUIRE(a.B >= 0 && a.nH > 0 && a.gh > 0 && a.gw > 0, "attn_relpos: bad shape");
   SF_REQUIRE(sm_scale > 0.f, "attn_relpos: sm_scale must be positive");
+  // an empty batch is a valid call that does nothing (its buffers may be null)
+  SF_REQUIRE(a.B == 0 || (a.q && a.k && a.v && a.out && a.rh && a.rw), "attn_relpos: null pointer");
   if (dtype != SAMFAST_BF16) SF_FAIL(SAMFAST_E_UNSUPPORTED, "attn_relpos: only bf16 is built");
   if (hd != 64 && hd != 80)
     SF_FAIL(SAMFAST_E_UNSUPPORTED, "attn_relpos: head_dim %d not in {64, 80}", hd);
@@ -932,6 +933,7 @@ static int attn_dispatch(bool fused, AttnArgs& a, int hd, int dtype, float sm_sc
                    a.rw_sh % 4 == 0 && a.rw_sn % 4 == 0,
                "attn_relpos: rel_w rows must be 8-byte aligned");
   }
+  if (a.B == 0) return SAMFAST_OK;
   a.c = sm_scale * kLog2e;
   a.inv_scale = 1.0f / sm_scale;
   if (hd == 64)

@@ -577,7 +577,8 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
                        int N, int K, hipStream_t stream, const void* residual = nullptr,
                        int64_t ld_res = 0, const int32_t* dst_row = nullptr,
                        int layout = SAMFAST_LAYOUT_ROWMAJOR) {
-  SF_REQUIRE(xq && wq && out, "gemm_i8: null pointer");
+  // no rows: nothing to do, and the row operands of an empty call may be null
+  SF_REQUIRE(wq && (M == 0 || (xq && out)), "gemm_i8: null pointer");
   SF_REQUIRE(layout == SAMFAST_LAYOUT_ROWMAJOR || layout == SAMFAST_LAYOUT_KB64, "gemm_i8: unknown layout %d", layout);
   SF_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_i8: bad shape M=%lld N=%d K=%d", (long long)M, N, K);
   SF_REQUIRE(M < (1ll << 31) - 256, "gemm_i8: M=%lld too large", (long long)M);
@@ -590,10 +591,15 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   if (epi == EPI_I32) {
     SF_REQUIRE(aligned16(out) && ldo % 4 == 0, "gemm_i8: int32 output must be 16-byte aligned rows");
   } else {
-    SF_REQUIRE(sx && sw, "gemm_i8: null scale pointer");
+    SF_REQUIRE(sw && (M == 0 || sx), "gemm_i8: null scale pointer");
     SF_REQUIRE(aligned16(out) && ldo % 8 == 0, "gemm_i8: bf16 output rows must be 16-byte aligned");
     SF_REQUIRE(aligned16(sw) && aligned16(sx) && (!bias || aligned16(bias)),
                "gemm_i8: sx / sw / bias must be 16-byte aligned");
+  }
+  if (epi == EPI_RESIDUAL_BF16) {
+    SF_REQUIRE((residual || M == 0) && aligned16(residual) && ld_res >= N && ld_res % 8 == 0,
+               "gemm_i8: residual must be non-null with 16-byte aligned rows");
+    SF_REQUIRE(!dst_row || aligned16(dst_row), "gemm_i8: dst_row must be 16-byte aligned");
   }
   if (M == 0) return SAMFAST_OK;
   GemmArgs a;
@@ -606,11 +612,6 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   }
   a.residual = reinterpret_cast<const unsigned short*>(residual);
   a.ld_res = ld_res; a.dst_row = dst_row;
-  if (epi == EPI_RESIDUAL_BF16) {
-    SF_REQUIRE(residual && aligned16(residual) && ld_res >= N && ld_res % 8 == 0,
-               "gemm_i8: residual must be non-null with 16-byte aligned rows");
-    SF_REQUIRE(!dst_row || aligned16(dst_row), "gemm_i8: dst_row must be 16-byte aligned");
-  }
   const char* force = getenv("SAMFAST_GEMM_TM");  // tuning aid: 2 or 4
   const bool generic_k = K / GBK < 4;  // fewer k tiles than LDS stages
   const int tm = generic_k ? 2 : (force && atoi(force) == 4 ? 4 : 2);

@@ -498,7 +498,8 @@ static int sparse_common(int epi, const int8_t* xq, const float* sx, const int8_
                          int64_t ldo, int64_t M, int N, int K, hipStream_t stream,
                          const void* residual = nullptr, int64_t ld_res = 0,
                          int layout = SAMFAST_LAYOUT_ROWMAJOR) {
-  SF_REQUIRE(xq && wc && widx && out, "gemm_i8_sparse24: null pointer");
+  // no rows: nothing to do, and the row operands of an empty call may be null
+  SF_REQUIRE(wc && widx && (M == 0 || (xq && out)), "gemm_i8_sparse24: null pointer");
   SF_REQUIRE(layout == SAMFAST_LAYOUT_ROWMAJOR || layout == SAMFAST_LAYOUT_KB64,
              "gemm_i8_sparse24: unknown layout %d", layout);
   SF_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_i8_sparse24: bad shape M=%lld N=%d K=%d", (long long)M, N, K);
@@ -514,11 +515,11 @@ static int sparse_common(int epi, const int8_t* xq, const float* sx, const int8_
   SF_REQUIRE(aligned16(xq) && aligned16(wc) && aligned16(widx) && aligned16(out),
              "gemm_i8_sparse24: operands and output must be 16-byte aligned");
   if (epi != SEPI_I32) {
-    SF_REQUIRE(sx && sw, "gemm_i8_sparse24: null scale pointer");
+    SF_REQUIRE(sw && (M == 0 || sx), "gemm_i8_sparse24: null scale pointer");
     SF_REQUIRE(aligned16(sw) && (!bias || aligned16(bias)), "gemm_i8_sparse24: sw / bias must be 16-byte aligned");
   }
   if (epi == SEPI_RESIDUAL)
-    SF_REQUIRE(residual && aligned16(residual) && ld_res >= N && ld_res % 8 == 0,
+    SF_REQUIRE((residual || M == 0) && aligned16(residual) && ld_res >= N && ld_res % 8 == 0,
                "gemm_i8_sparse24: residual must be non-null with 16-byte aligned rows");
   if (M == 0) return SAMFAST_OK;
   SparseArgs a;

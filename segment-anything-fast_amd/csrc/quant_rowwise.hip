@@ -267,8 +267,8 @@ static int check_common(const char* who, const void* x, int64_t ldx, const int8_
                         int64_t M, int K, int dtype, int layout) {
   SF_REQUIRE(layout == SAMFAST_LAYOUT_ROWMAJOR || (layout == SAMFAST_LAYOUT_KB64 && K % 64 == 0),
              "%s: layout must be row-major, or K-block major with K %% 64 == 0", who);
-  SF_REQUIRE(x && xq && sx, "%s: null pointer", who);
   SF_REQUIRE(M >= 0 && K > 0, "%s: bad shape M=%lld K=%d", who, (long long)M, K);
+  SF_REQUIRE(M == 0 || (x && xq && sx), "%s: null pointer", who);  // no rows: the buffers may be null
   if (dtype != SAMFAST_BF16) SF_FAIL(SAMFAST_E_UNSUPPORTED, "%s: only bf16 input", who);
   SF_REQUIRE(K % 8 == 0 && K <= 8192, "%s: K=%d must be a multiple of 8, <= 8192", who, K);
   SF_REQUIRE(ldx >= K && ldx % 8 == 0, "%s: ldx=%lld must be >= K and a multiple of 8", who,

@@ -33,6 +33,36 @@ def test_library_exports_every_declared_symbol():
     assert loaded.samfast_arch() == b"gfx950"
 
 
+def test_empty_calls_are_no_ops_without_gpu():
+    """No rows / no images: every entry point validates the shape, launches nothing and returns 0,
+    also with null row buffers (what an empty tensor hands over); a negative count is an error."""
+    from samfast_amd import _lib
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    p += (-p) % 16
+    assert lib.samfast_quant_rowwise_i8(None, 256, None, None, 0, 256, 0, 0, None) == 0
+    assert lib.samfast_quant_rowwise_i8(None, 256, None, None, 0, 256, 0, 1, None) == 0
+    assert lib.samfast_layernorm_quant_i8(None, 256, p, p, 1e-6, None, None, None, 0, 256, 0, 0, None) == 0
+    assert lib.samfast_gemm_i8_i32(None, p, None, 0, 64, 256, None) == 0
+    assert lib.samfast_gemm_i8_scale_bias(None, None, p, p, None, None, 64, 0, 64, 256, 0, None) == 0
+    assert lib.samfast_gemm_i8_fused(None, None, p, p, p, None, 64, 0, 64, 256, 0, 2, None, 64, None, 1, None) == 0
+    assert lib.samfast_gemm_i8_sparse24_i32(None, p, p, None, 0, 64, 256, None) == 0
+    assert lib.samfast_gemm_i8_sparse24_fused(None, None, p, p, p, None, None, 64, 0, 64, 256, 0, 1, None, 0, 0, None) == 0
+    strides = [64] * 12
+    assert lib.samfast_attn_relpos_fwd(None, None, None, None, None, None, 0, 12, 64, 64, 64,
+                                       *strides, 0, 0.125, None) == 0
+    assert lib.samfast_attn_relpos_bias_fwd(None, None, None, None, None, None, 0, 12, 14, 14, 80,
+                                            *([80] * 12), *([16] * 6), 0, 0.1, None) == 0
+    # the shape is still checked
+    assert lib.samfast_quant_rowwise_i8(None, 256, None, None, -1, 256, 0, 0, None) == -1
+    assert lib.samfast_gemm_i8_i32(None, p, None, 0, 64, 100, None) == -1
+    assert lib.samfast_attn_relpos_fwd(None, None, None, None, None, None, 0, 12, 64, 64, 48,
+                                       *strides, 0, 0.125, None) == -2
+    assert lib.samfast_attn_relpos_fwd(None, None, None, None, None, None, -1, 12, 64, 64, 64,
+                                       *strides, 0, 0.125, None) == -1
+
+
 def test_argument_validation_without_gpu():
     """Validation runs on the host before any launch, so error codes are testable here."""
     from samfast_amd import _lib

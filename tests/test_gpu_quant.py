@@ -270,3 +270,43 @@ def test_kblock_major_layout_matches_row_major(M, N, K):
                                         layout=_lib.LAYOUT_KB64)
         torch.cuda.synchronize()
         assert torch.equal(y0.view(torch.int16), y1.view(torch.int16))
+
+
+def test_empty_inputs_give_empty_outputs():
+    """No rows and no images: every operator returns a correctly shaped empty result (the calls go
+    through the C ABI, which launches nothing)."""
+    from samfast_amd import _lib, ops
+    dev = "cuda"
+    K, N = 256, 64
+    x = torch.empty((0, K), dtype=torch.bfloat16, device=dev)
+    wq = torch.ones((N, K), dtype=torch.int8, device=dev)
+    sw = torch.ones(N, device=dev)
+    bias = torch.zeros(N, device=dev)
+    for layout in (_lib.LAYOUT_ROWMAJOR, _lib.LAYOUT_KB64):
+        xq, sx = ops.quant_rowwise(x, layout)
+        assert xq.numel() == 0 and sx.shape == (0,)
+        g = torch.ones(K, dtype=torch.bfloat16, device=dev)
+        lq, ls = ops.layernorm_quant(x, g, torch.zeros_like(g), 1e-6, layout=layout)
+        assert lq.numel() == 0 and ls.shape == (0,)
+        w = ops.to_kb64(wq) if layout == _lib.LAYOUT_KB64 else wq
+        for epi in (_lib.EPILOGUE_NONE, _lib.EPILOGUE_GELU):
+            y = ops.gemm_i8_fused(xq, sx, w, sw, bias, epi, layout=layout)
+            assert y.shape == (0, N) and y.dtype == torch.bfloat16
+        res = torch.empty((0, N), dtype=torch.bfloat16, device=dev)
+        y = ops.gemm_i8_fused(xq, sx, w, sw, bias, _lib.EPILOGUE_RESIDUAL, residual=res, layout=layout)
+        assert y.shape == (0, N)
+    xq, sx = ops.quant_rowwise(x)
+    assert ops.gemm_i8_i32(xq, wq).shape == (0, N)
+    assert ops.gemm_i8_scale_bias(xq, sx, wq, sw, None).shape == (0, N)
+    wc, widx = ops.prune24_pack(wq)
+    assert ops.gemm_i8_sparse24_i32(xq, wc, widx).shape == (0, N)
+    assert ops.gemm_i8_sparse24_fused(xq, sx, wc, widx, sw, bias, _lib.EPILOGUE_GELU).shape == (0, N)
+    for (gh, gw, hd) in ((64, 64, 80), (14, 14, 64)):
+        q = torch.empty((0, 2, gh * gw, hd), dtype=torch.bfloat16, device=dev)
+        rph = torch.zeros((2 * gh - 1, hd), dtype=torch.bfloat16, device=dev)
+        rpw = torch.zeros((2 * gw - 1, hd), dtype=torch.bfloat16, device=dev)
+        assert ops.attn_relpos(q, q, q, rph, rpw, (gh, gw)).shape == q.shape
+        rel_h = torch.empty((0, 2, gh * gw, gh), dtype=torch.bfloat16, device=dev)
+        rel_w = torch.empty((0, 2, gh * gw, gw), dtype=torch.bfloat16, device=dev)
+        assert ops.attn_relpos_bias(q, q, q, rel_h, rel_w).shape == q.shape
+    torch.cuda.synchronize()
