@@ -195,7 +195,7 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
           const float d0 = f[i][2 * j] - mean, d1 = f[i][2 * j + 1] - mean;
           f[i][2 * j] = d0;
           f[i][2 * j + 1] = d1;
-          s2 += d0 * d0 + d1 * d1;
+          s2 = fmaf(d1, d1, fmaf(d0, d0, s2));
         }
       }
     }
@@ -207,8 +207,9 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
         const in_t g = gw[i], b = bw[i];
 #pragma unroll
         for (int j = 0; j < W; ++j) {
-          const float y0 = f[i][2 * j] * rstd * bf16_lo_to_f32(g[j]) + bf16_lo_to_f32(b[j]);
-          const float y1 = f[i][2 * j + 1] * rstd * bf16_hi_to_f32(g[j]) + bf16_hi_to_f32(b[j]);
+          // (x - mean) * rstd, then one fused multiply-add with gamma and beta
+          const float y0 = fmaf(f[i][2 * j] * rstd, bf16_lo_to_f32(g[j]), bf16_lo_to_f32(b[j]));
+          const float y1 = fmaf(f[i][2 * j + 1] * rstd, bf16_hi_to_f32(g[j]), bf16_hi_to_f32(b[j]));
           const unsigned int y = pack_bf16x2(y0, y1);  // the bf16 values a separate LayerNorm would have stored
           f[i][2 * j] = bf16_lo_to_f32(y);
           f[i][2 * j + 1] = bf16_hi_to_f32(y);
