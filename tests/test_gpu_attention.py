@@ -245,3 +245,25 @@ def test_reference_test_recipe_against_sdpa(batch, head, hidden_dim):
         ref = torch.nn.functional.scaled_dot_product_attention(
             q[b:b + 1].float(), k[b:b + 1].float(), v[b:b + 1].float(), attn_mask=bias)
         torch.testing.assert_close(ref.to(dtype), out[b:b + 1], rtol=1e-3, atol=1e-3)
+
+
+def test_seeded_sweep_of_window_and_grid_shapes():
+    """Random window shapes up to the kernel's limits (gh <= 15, gw <= 16, <= 208 tokens) and 64-wide
+    grids with an even number of rows, both head sizes, against the fp32 oracle at the stated bar."""
+    import numpy as np
+    from samfast_amd import ops
+    rng = np.random.default_rng(31)
+    shapes = []
+    while len(shapes) < 14:
+        gh, gw = int(rng.integers(1, 16)), int(rng.integers(1, 17))
+        if gh * gw <= 208:
+            shapes.append((int(rng.integers(1, 7)), int(rng.integers(1, 5)), gh, gw, (64, 80)[len(shapes) % 2]))
+    for gh in (2, 6, 10, 30):
+        shapes.append((int(rng.integers(1, 3)), int(rng.integers(1, 3)), gh, 64, (64, 80)[(gh // 2) % 2]))
+    for case, (B, nH, gh, gw, hd) in enumerate(shapes):
+        print(f"case attention sweep {case}: B={B} nH={nH} grid={gh}x{gw} hd={hd}", flush=True)
+        q, k, v, rph, rpw = attn_inputs(B, nH, gh, gw, hd, seed=300 + case)
+        ref = _oracle_tables(q, k, v, rph, rpw, (gh, gw))
+        out = ops.attn_relpos(q.cuda(), k.cuda(), v.cuda(), rph.cuda(), rpw.cuda(), (gh, gw))
+        torch.cuda.synchronize()
+        _check(out, ref, f"sweep {B}x{nH}x{gh}x{gw}x{hd}")

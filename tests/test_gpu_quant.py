@@ -310,3 +310,33 @@ def test_empty_inputs_give_empty_outputs():
         rel_w = torch.empty((0, 2, gh * gw, gw), dtype=torch.bfloat16, device=dev)
         assert ops.attn_relpos_bias(q, q, q, rel_h, rel_w).shape == q.shape
     torch.cuda.synchronize()
+
+
+def test_seeded_sweep_of_ragged_shapes_bit_exact():
+    """Thirty random shapes (ragged rows, column counts that are not multiples of the 256-wide tile,
+    every K the kernels accept in steps of 64) - quantiser codes and scales, int32 accumulators and
+    the fused scale-and-bias output in both operand layouts, all bit-exact against the oracle."""
+    from samfast_amd import _lib, ops
+    rng = np.random.default_rng(2024)
+    for case in range(30):
+        M = int(rng.integers(1, 700))
+        N = 8 * int(rng.integers(1, 90))
+        K = 64 * int(rng.integers(1, 24))
+        print(f"case sweep {case}: M={M} N={N} K={K}", flush=True)
+        x, w, b = linear_inputs(M, K, N, seed=1000 + case)
+        xq_ref, sx_ref = orq.quantize_rows_absmax(x)
+        wq_ref, sw_ref = orq.quantize_rows_absmax(w.float())
+        xq, sx = ops.quant_rowwise(x.cuda())
+        assert np.array_equal(xq.cpu().numpy(), xq_ref) and np.array_equal(sx.cpu().numpy(), sx_ref)
+        wq = torch.from_numpy(wq_ref).cuda()
+        sw = torch.from_numpy(sw_ref).cuda()
+        acc_ref = orq.int8_gemm_i64(xq_ref, wq_ref)
+        acc = ops.gemm_i8_i32(xq, wq)
+        assert np.array_equal(acc.cpu().numpy().astype(np.int64), acc_ref)
+        y_ref = orq.scale_bias_epilogue(acc_ref.astype(np.int32), sx_ref, sw_ref, b.float().numpy())
+        bias = b.float().cuda()
+        y = ops.gemm_i8_fused(xq, sx, wq, sw, bias, _lib.EPILOGUE_NONE)
+        assert torch.equal(y.cpu().view(torch.int16), y_ref.view(torch.int16))
+        xk, _ = ops.quant_rowwise(x.cuda(), _lib.LAYOUT_KB64)
+        yk = ops.gemm_i8_fused(xk, sx, ops.to_kb64(wq), sw, bias, _lib.EPILOGUE_NONE, layout=_lib.LAYOUT_KB64)
+        assert torch.equal(yk.cpu().view(torch.int16), y_ref.view(torch.int16))

@@ -160,3 +160,23 @@ def test_apply_sparse_mlp_only_module_and_encoder():
     cos = torch.nn.functional.cosine_similarity(out.flatten(1), ref.flatten(1), dim=1).min().item()
     print(f"sparse mlp slice: cosine {cos:.6f}", flush=True)
     assert torch.isfinite(out).all() and cos >= 0.999, cos
+
+
+def test_seeded_sweep_of_ragged_shapes_sparse_bit_exact():
+    """Twenty random shapes: the 2:4 GEMM's accumulators equal the dense product with the pruned
+    int8 matrix bit for bit (K in steps of 128 from 256, as the sparse kernel requires)."""
+    from samfast_amd import ops
+    rng = np.random.default_rng(77)
+    for case in range(20):
+        M = int(rng.integers(1, 600))
+        N = 8 * int(rng.integers(1, 80))
+        K = 128 * int(rng.integers(2, 12))
+        print(f"case sparse sweep {case}: M={M} N={N} K={K}", flush=True)
+        g = torch.Generator().manual_seed(500 + case)
+        xq = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+        wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+        wc, widx = ops.prune24_pack(wq.cuda())
+        dense = orq.unpack_2_of_4(wc.cpu().numpy(), widx.cpu().numpy())
+        ref = orq.int8_gemm_i64(xq.numpy(), dense)
+        acc = ops.gemm_i8_sparse24_i32(xq.cuda(), wc, widx)
+        assert np.array_equal(acc.cpu().numpy().astype(np.int64), ref)
