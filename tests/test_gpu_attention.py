@@ -132,7 +132,9 @@ def test_unsupported_shapes_raise():
         ops.attn_relpos(q, q, q, t, t, (10, 10))
 
 
-@pytest.mark.parametrize("B,nH,H,W,ws,hd", [(2, 3, 20, 17, 14, 64), (1, 2, 64, 64, 14, 80), (2, 2, 9, 9, 3, 64)])
+@pytest.mark.parametrize("B,nH,H,W,ws,hd", [(2, 3, 20, 17, 14, 64), (1, 2, 64, 64, 14, 80), (2, 2, 9, 9, 3, 64),
+                                           (1, 1, 14, 14, 14, 80), (1, 2, 15, 29, 7, 64), (3, 1, 27, 13, 13, 80),
+                                           (1, 4, 1, 40, 14, 64), (2, 1, 33, 2, 11, 80)])
 def test_windowed_on_image_tokens_equals_partitioned_windows(B, nH, H, W, ws, hd):
     """samfast_attn_relpos_windowed_fwd = window_partition + per-window attention +
     window_unpartition: same bits as running the window kernel on explicitly partitioned,
