@@ -156,7 +156,7 @@ def _oracle_ln_quant(x, gamma, beta, eps, src_row=None):
     return orq.quantize_rows_absmax(y)
 
 
-@pytest.mark.parametrize("R,K", [(64, 768), (300, 1280), (50, 1024)])
+@pytest.mark.parametrize("R,K", [(64, 768), (300, 1280), (50, 1024), (7, 64), (33, 3072), (129, 5120), (5, 8192)])
 def test_layernorm_quant_vs_oracle(R, K):
     """LayerNorm is floating point (reduction order differs from the CPU), so codes may
     differ by one step where the normalised value sits on a rounding boundary:
