@@ -340,3 +340,23 @@ def test_seeded_sweep_of_ragged_shapes_bit_exact():
         xk, _ = ops.quant_rowwise(x.cuda(), _lib.LAYOUT_KB64)
         yk = ops.gemm_i8_fused(xk, sx, ops.to_kb64(wq), sw, bias, _lib.EPILOGUE_NONE, layout=_lib.LAYOUT_KB64)
         assert torch.equal(yk.cpu().view(torch.int16), y_ref.view(torch.int16))
+
+
+def test_quantiser_exact_ties_round_to_even():
+    """Rows whose scale is exactly 1 (absmax 127) and whose values sit exactly on half-integers: the
+    codes must be the even neighbours, as the oracle's (and IEEE's) round-half-to-even gives; and
+    rows with other scales carrying the same pattern, against the oracle."""
+    from samfast_amd import ops
+    K = 256
+    halves = torch.arange(0, 64, dtype=torch.float32) + 0.5          # 0.5 .. 63.5: exact in bf16
+    row = torch.cat([torch.tensor([127.0]), halves, -halves, torch.zeros(K - 129)])
+    x = torch.stack([row, row * 2.0, row * 0.75, row * 3.0, -row]).to(torch.bfloat16)
+    assert torch.equal(x[0].float(), row)                              # nothing was rounded away
+    xq_ref, sx_ref = orq.quantize_rows_absmax(x)
+    xq, sx = ops.quant_rowwise(x.cuda())
+    assert np.array_equal(sx.cpu().numpy(), sx_ref)
+    assert np.array_equal(xq.cpu().numpy(), xq_ref)
+    got = xq[0, 1:65].cpu().numpy()
+    expect = np.array([int(np.rint(k + 0.5)) for k in range(64)])     # numpy rint: half to even
+    assert sx_ref[0] == np.float32(1.0) and np.array_equal(got, expect) and got[0] == 0 and got[1] == 2 and got[2] == 2
+    assert np.array_equal(xq[0, 65:129].cpu().numpy(), -expect)
