@@ -33,9 +33,9 @@ extern "C" {
 
 #define SAMFAST_VERSION 1
 
-/* element types of attention operands / linear outputs */
+/* element type of attention operands / linear outputs: bf16 is the only one built (other
+ * values of a `dtype` argument return SAMFAST_E_UNSUPPORTED) */
 #define SAMFAST_BF16 0
-#define SAMFAST_F16 1
 
 #define SAMFAST_OK 0
 #define SAMFAST_E_INVALID (-1)      /* bad shape / stride / alignment / null pointer */
@@ -96,7 +96,7 @@ int samfast_attn_relpos_fwd(
  * the reference's zero-padded tokens: they take part as keys / values with the rows
  * pad_k / pad_v ((nH, hd) each, same element type - for SAM the bf16-rounded k and v bias of
  * the qkv Linear, which is what a zero input row produces) and produce no output.
- * rel_pos_h / rel_pos_w: (2*ws-1, hd).  Supported: hd in {64, 80}, ws <= 14, bf16.
+ * rel_pos_h / rel_pos_w: (2*ws-1, hd).  Supported: hd in {64, 80}, ws <= 14 (ws*ws <= 208), bf16.
  */
 int samfast_attn_relpos_windowed_fwd(
     const void* q, const void* k, const void* v,
@@ -138,6 +138,9 @@ int samfast_attn_relpos_bias_fwd(
  * activation quantiser torchao.apply_dynamic_quant installs in front of every
  * Linear (call site experiments/eval_combo.py:357-359).  K % 8 == 0, K <= 8192.
  * `layout` is the layout xq is written in (SAMFAST_LAYOUT_*).
+ * A row that holds a NaN gets sx = NaN (its codes are unspecified), so the Linear that
+ * consumes it returns NaN for that row and only that row; an infinite value makes the
+ * scale infinite.  The same holds for samfast_layernorm_quant_i8.
  */
 int samfast_quant_rowwise_i8(
     const void* x, int64_t ldx, int8_t* xq, float* sx,

@@ -54,28 +54,32 @@ def quantize_rows_absmax(x):
     experiments/eval_combo.py:357-359) and, applied to a (N, K) weight, for
     its per-output-channel weight quantiser.
     """
-    xf = _to_f32_numpy(x)
-    assert xf.ndim == 2
-    absmax = np.maximum(np.abs(xf).max(axis=1), EPS).astype(np.float32)
-    scale = (absmax / QMAX).astype(np.float32)
-    ratio = (xf / scale[:, None]).astype(np.float32)
-    q = np.clip(np.rint(ratio), -127.0, 127.0).astype(np.int8)  # rint = half to even
-    return q, scale
+    xf = x.detach().to(torch.float32) if isinstance(x, torch.Tensor) else torch.from_numpy(_to_f32_numpy(x))
+    assert xf.dim() == 2
+    # torch's CPU element-wise kernels: one IEEE fp32 operation per call (several threads);
+    # amax propagates a NaN, round() is round-half-to-even
+    absmax = xf.abs().amax(dim=1).clamp_min(float(EPS))
+    scale = absmax / float(QMAX)
+    ratio = xf / scale[:, None]
+    q = ratio.round().clamp_(-127.0, 127.0).to(torch.int8)
+    return q.numpy(), scale.numpy()
 
 
 def int8_gemm_i32(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:
     """acc[m, n] = sum_k xq[m, k] * wq[n, k] as int32 (torch._int_mm semantics).
 
-    |acc| <= K * 127^2 < 2^31 for K <= 133 000, so int32 never wraps here.
+    |acc| <= K * 128^2 < 2^31 for K <= 131 000, so int32 never wraps here.  Large
+    products run as a float64 matrix product on the BLAS threads: every product and
+    every partial sum is an integer far below 2^53, so the result is exact whatever
+    the summation order (torch._int_mm on a CPU gives the same numbers 50x slower;
+    tests/test_oracle_quant.py checks the two and the int64 product against each other).
     """
     assert xq.dtype == np.int8 and wq.dtype == np.int8
     M, K = xq.shape
-    N = wq.shape[0]
-    if M > 16 and K % 8 == 0 and N % 8 == 0:
-        # torch._int_mm is multi-threaded; exact for integers like any other route.
-        a = torch.from_numpy(np.ascontiguousarray(xq))
-        b = torch.from_numpy(np.ascontiguousarray(wq)).t()
-        return torch._int_mm(a, b).numpy()
+    if M * wq.shape[0] * K >= 1 << 22:
+        a = torch.from_numpy(np.ascontiguousarray(xq)).to(torch.float64)
+        b = torch.from_numpy(np.ascontiguousarray(wq)).to(torch.float64)
+        return (a @ b.t()).to(torch.int32).numpy()
     return (xq.astype(np.int32) @ wq.astype(np.int32).T).astype(np.int32)
 
 
@@ -85,13 +89,14 @@ def int8_gemm_i64(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:
 
 
 def scale_bias_epilogue(acc: np.ndarray, sx: np.ndarray, sw: np.ndarray, bias) -> torch.Tensor:
-    """y = (float(acc) * sx[m]) * sw[n] + bias[n], each step one fp32 op, -> bf16."""
-    t = acc.astype(np.float32)  # int32 -> fp32, round to nearest even
-    t = (t * sx.astype(np.float32)[:, None]).astype(np.float32)
-    t = (t * sw.astype(np.float32)[None, :]).astype(np.float32)
+    """y = (float(acc) * sx[m]) * sw[n] + bias[n], each step one fp32 op, -> bf16.
+    (torch's CPU element-wise kernels: one IEEE operation per call, several threads.)"""
+    t = torch.from_numpy(np.ascontiguousarray(acc)).to(torch.float32)  # int32 -> fp32, round to nearest even
+    t = t * torch.from_numpy(np.ascontiguousarray(sx, dtype=np.float32))[:, None]
+    t = t * torch.from_numpy(np.ascontiguousarray(sw, dtype=np.float32))[None, :]
     if bias is not None:
-        t = (t + _to_f32_numpy(bias)[None, :]).astype(np.float32)
-    return torch.from_numpy(t).to(torch.bfloat16)
+        t = t + torch.from_numpy(_to_f32_numpy(bias))[None, :]
+    return t.to(torch.bfloat16)
 
 
 def dynamic_int8_linear(x: torch.Tensor, weight: torch.Tensor, bias) -> torch.Tensor:

@@ -75,21 +75,27 @@ SF_DEVICE float wave_max_nonneg(float v) {
 // Rounding: adding 1.5 * 2^23 to r (|r| <= 127) leaves rint(r) - half to even - in the low
 // mantissa bits, so the low byte of the sum's bit pattern is the int8 code; subtracting the
 // constant again gives rint(r) as a float for the near-tie test.
+// Returns true when the chunk holds a NaN: the comparison that finds near-ties is written so
+// that a NaN product also takes the slow path, where the chunk's values are looked at once more;
+// the common path pays nothing for it.
 template <int EPC>
-SF_DEVICE void quantize_chunk(const float (&v)[EPC], float scale, float inv_scale, unsigned int (&out)[EPC / 4]) {
+SF_DEVICE bool quantize_chunk(const float (&v)[EPC], float scale, float inv_scale, unsigned int (&out)[EPC / 4]) {
   constexpr float kMagic = 12582912.0f;  // 1.5 * 2^23
   float m[EPC];
-  bool near_tie = false;
+  bool near_tie = false, saw_nan = false;
 #pragma unroll
   for (int e = 0; e < EPC; ++e) {
     const float r = v[e] * inv_scale;
     m[e] = r + kMagic;
     const float d = r - (m[e] - kMagic);  // r - rint(r), exact
-    near_tie |= fabsf(d) > 0.5f - 1e-4f;
+    near_tie |= !(fabsf(d) <= 0.5f - 1e-4f);  // also true for a NaN
   }
   if (near_tie) {
 #pragma unroll
-    for (int e = 0; e < EPC; ++e) m[e] = v[e] / scale + kMagic;  // IEEE division
+    for (int e = 0; e < EPC; ++e) {
+      m[e] = v[e] / scale + kMagic;  // IEEE division
+      saw_nan |= v[e] != v[e];
+    }
   }
 #pragma unroll
   for (int g = 0; g < EPC / 4; ++g) {
@@ -100,6 +106,7 @@ SF_DEVICE void quantize_chunk(const float (&v)[EPC], float scale, float inv_scal
     const unsigned int hi = __builtin_amdgcn_perm(w3, w2, 0x04000c0cu);  // [0, 0, w2.b0, w3.b0]
     out[g] = lo | hi;
   }
+  return saw_nan;
 }
 
 // A lane holds chunks lane, lane + 64, ... of EPC elements (NCH of them: K <= NCH * 64 * EPC).
@@ -227,17 +234,21 @@ __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_k
 
   const float scale = fmaxf(amax, 1e-5f) / 127.0f;
   const float inv_scale = 1.0f / scale;
-  if (lane == 0) a.sx[row] = scale;
 
+  bool saw_nan = false;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = lane + i * 64;
     if (c < nchunk) {
       unsigned int codes[EPC / 4];
-      quantize_chunk<EPC>(f[i], scale, inv_scale, codes);
+      saw_nan |= quantize_chunk<EPC>(f[i], scale, inv_scale, codes);
       store_chunk(c, codes);
     }
   }
+  // the maximum above drops NaNs (fmaxf returns its other operand); a row that holds one gets a
+  // NaN scale, so that the Linear reading it returns NaN for this row as a float Linear would
+  const bool row_nan = __any(saw_nan);
+  if (lane == 0) a.sx[row] = row_nan ? __uint_as_float(0x7fc00000u) : scale;
 }
 
 template <int NCH, int EPC, bool LN>

@@ -52,6 +52,14 @@ def _custom_flash_aligned_gpu(q, k, v, rel_h_w, sm_scale):
     assert q.shape == k.shape == v.shape
     assert rel_h_w.shape[-1] == 128 and rel_h_w.shape[-2] == q.shape[-2]
     assert rel_h_w.dtype == q.dtype
+    # key n sits at grid row n // 64, column n % 64 (flash_4.py:115-116): N / 64 key rows, of
+    # which the first N / 64 columns of the rel_h half are the ones the kernel reads
+    N = q.shape[-2]
+    if N % 128 != 0 or N // 64 > 64:
+        raise RuntimeError(
+            f"customflash::custom_flash_aligned: {N} tokens are not a 64-wide key grid of at most 64 "
+            "rows (an even number of them)")
+    gh = N // 64
     if rel_h_w.stride(-1) != 1:
         rel_h_w = rel_h_w.contiguous()
     if q.stride(-1) != 1:
@@ -60,7 +68,7 @@ def _custom_flash_aligned_gpu(q, k, v, rel_h_w, sm_scale):
         k = k.contiguous()
     if v.stride(-1) != 1:
         v = v.contiguous()
-    return ops.attn_relpos_bias(q, k, v, rel_h_w[..., :64], rel_h_w[..., 64:], sm_scale)
+    return ops.attn_relpos_bias(q, k, v, rel_h_w[..., :gh], rel_h_w[..., 64:], sm_scale)
 
 
 if _OWNS_SCHEMA:

@@ -133,6 +133,7 @@ class Block(nn.Module):
                 and self.norm1.elementwise_affine and self.norm2.elementwise_affine
                 and self.norm1.bias is not None and self.norm2.bias is not None
                 and self.norm1.weight.dtype == torch.bfloat16
+                and attn.rel_pos_h.dtype == torch.bfloat16 and attn.rel_pos_w.dtype == torch.bfloat16
                 and isinstance(mlp.act, nn.GELU) and getattr(mlp.act, "approximate", "none") == "none"):
             return False
         B, H, W, C = x.shape
@@ -359,7 +360,7 @@ class PatchEmbed(nn.Module):
             # output is already (B, H, W, C)
             B, C, H, W = x.shape
             gh, gw = H // kh, W // kw
-            cols = x.view(B, C, gh, kh, gw, kw).permute(0, 2, 4, 1, 3, 5).reshape(B * gh * gw, C * kh * kw)
-            y = F.linear(cols, p.weight.view(p.out_channels, C * kh * kw), p.bias)
+            cols = x.reshape(B, C, gh, kh, gw, kw).permute(0, 2, 4, 1, 3, 5).reshape(B * gh * gw, C * kh * kw)
+            y = F.linear(cols, p.weight.reshape(p.out_channels, C * kh * kw), p.bias)
             return y.view(B, gh, gw, p.out_channels)
         return self.proj(x).permute(0, 2, 3, 1)

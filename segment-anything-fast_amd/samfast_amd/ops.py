@@ -79,9 +79,21 @@ def _bnhd_strides(t: torch.Tensor) -> Tuple[int, int, int]:
 def _dtype_code(t: torch.Tensor) -> int:
     if t.dtype == torch.bfloat16:
         return _lib.SAMFAST_BF16
-    if t.dtype == torch.float16:
-        return _lib.SAMFAST_F16
-    raise RuntimeError(f"samfast: unsupported dtype {t.dtype}")
+    raise RuntimeError(f"samfast: unsupported dtype {t.dtype} (the kernels are built for bfloat16)")
+
+
+def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: Optional[torch.Tensor],
+               tokens: int) -> None:
+    """The library only receives the grid: it walks `tokens` rows of every (batch, head)
+    slice whatever the tensors hold, so their shapes are pinned here, before any launch."""
+    if q.dim() != 4 or q.shape[2] != tokens:
+        raise RuntimeError(f"samfast: q must be (B, nH, {tokens}, hd) for this grid, got {tuple(q.shape)}")
+    if k.shape != q.shape or v.shape != q.shape:
+        raise RuntimeError("samfast: k and v must have the shape of q")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError("samfast: k and v must have the dtype of q")
+    if out is not None and (out.shape != q.shape or out.dtype != q.dtype or out.device != q.device):
+        raise RuntimeError("samfast: out must have the shape, dtype and device of q")
 
 
 def attn_supported(N: int, grid_hw: Tuple[int, int], hd: int, dtype: torch.dtype) -> bool:
@@ -103,9 +115,10 @@ def attn_relpos(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     token strides (head_dim contiguous).  Returns (B, nH, N, hd) laid out
     token-major, i.e. as a (B, N, nH*hd) buffer viewed head-major, unless `out`
     is given."""
+    gh, gw = grid_hw
+    _check_qkv(q, k, v, out, gh * gw)
     _require_gpu(q, k, v, rel_pos_h, rel_pos_w)
     B, nH, N, hd = q.shape
-    gh, gw = grid_hw
     if out is None:
         out = torch.empty((B, N, nH, hd), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
     rel_pos_h = rel_pos_h.contiguous()
@@ -134,13 +147,15 @@ def attn_relpos_windowed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     """Windowed attention on image-ordered tokens (partition + attention + unpartition).
     q, k, v: (B, nH, H*W, hd) views with contiguous hd; pad_k / pad_v: (nH, hd) rows standing
     for the zero-padded tokens.  Returns (B, H*W, nH, hd) contiguous."""
+    H, W = grid_hw
+    _check_qkv(q, k, v, None, H * W)
     _require_gpu(q, k, v, rel_pos_h, rel_pos_w, pad_k, pad_v)
     B, nH, N, hd = q.shape
-    H, W = grid_hw
-    if H * W != N:
-        raise RuntimeError("samfast: grid does not match the token count")
     if tuple(rel_pos_h.shape) != (2 * window - 1, hd) or tuple(rel_pos_w.shape) != (2 * window - 1, hd):
         raise RuntimeError("samfast: rel_pos tables must be (2*window-1, head_dim)")
+    # the kernel reads the tables as q's element type
+    rel_pos_h = rel_pos_h.to(q.dtype).contiguous()
+    rel_pos_w = rel_pos_w.to(q.dtype).contiguous()
     for t in (pad_k, pad_v):
         if tuple(t.shape) != (nH, hd) or not t.is_contiguous() or t.dtype != q.dtype:
             raise RuntimeError("samfast: pad_k / pad_v must be contiguous (nH, hd) tensors of q's dtype")
@@ -152,8 +167,8 @@ def attn_relpos_windowed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     code = _timed(
         "attn_window", 4.0 * nwin * nH * nt * nt * hd, "flop",
         lambda: lib.samfast_attn_relpos_windowed_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), rel_pos_h.contiguous().data_ptr(),
-            rel_pos_w.contiguous().data_ptr(), pad_k.data_ptr(), pad_v.data_ptr(), out.data_ptr(),
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), rel_pos_h.data_ptr(),
+            rel_pos_w.data_ptr(), pad_k.data_ptr(), pad_v.data_ptr(), out.data_ptr(),
             B, nH, H, W, window, hd,
             *_bnhd_strides(q), *_bnhd_strides(k), *_bnhd_strides(v), *_bnhd_strides(o),
             _dtype_code(q), float(scale), _stream()))
@@ -168,11 +183,14 @@ def attn_relpos_bias(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     """Same attention with caller-computed bias factors rel_h (B, nH, N, gh) and
     rel_w (B, nH, N, gw) (last axis contiguous).  Returns a contiguous
     (B, nH, N, hd) tensor unless `out` is given."""
-    _require_gpu(q, k, v, rel_h, rel_w)
-    B, nH, N, hd = q.shape
     gh, gw = rel_h.shape[-1], rel_w.shape[-1]
+    _check_qkv(q, k, v, out, gh * gw)
+    B, nH, N, hd = q.shape
+    if tuple(rel_h.shape) != (B, nH, N, gh) or tuple(rel_w.shape) != (B, nH, N, gw):
+        raise RuntimeError("samfast: bias factors must be (B, nH, N, gh) and (B, nH, N, gw) with gh*gw == N")
     if rel_h.dtype != q.dtype or rel_w.dtype != q.dtype:
         raise RuntimeError("samfast: bias factors must have the dtype of q")
+    _require_gpu(q, k, v, rel_h, rel_w)
     if out is None:
         out = torch.empty((B, nH, N, hd), dtype=q.dtype, device=q.device)
     scale = float(sm_scale) if sm_scale is not None else 1.0 / math.sqrt(hd)

@@ -27,14 +27,39 @@ from ._lib import EPILOGUE_NONE, LAYOUT_KB64, LAYOUT_ROWMAJOR
 from .tools import replace_with_custom_fn_if_matches_filter
 
 
-def quantize_weight_per_channel(weight: torch.Tensor):
-    """(N, K) float -> (int8 (N, K), fp32 scale (N,)), scale = max(absmax, 1e-5)/127,
-    q = clamp(rint(w / scale), -127, 127).  fp32 arithmetic, done once at swap time."""
-    w = weight.detach().to(torch.float32)
-    absmax = w.abs().amax(dim=1).clamp_min(1e-5)
-    scale = absmax / 127.0
-    q = torch.round(w / scale[:, None]).clamp_(-127, 127).to(torch.int8)
-    return q.contiguous(), scale.contiguous()
+WEIGHT_CONVENTIONS = ("absmax127", "torchao")
+
+
+def quantize_weight_per_channel(weight: torch.Tensor, convention: str = "absmax127"):
+    """(N, K) float -> (int8 (N, K), fp32 scale (N,)), done once at swap time.
+
+    "absmax127" (default): fp32 arithmetic, scale = max(absmax, 1e-5) / 127,
+        q = clamp(rint(w / scale), -127, 127) - the symmetric convention of the activation
+        quantiser; codes never reach -128.
+    "torchao": torchao's `dynamically_quantize_per_channel(w, -128, 127, torch.int8)` as its
+        apply_dynamic_quant runs it on the weight (call site experiments/eval_combo.py:357-359),
+        restated from the published routine: scale = max(absmax / 127.5, eps) with eps = float32
+        machine epsilon (the symmetric range is split as (quant_max - quant_min) / 2), the scale
+        is stored in the WEIGHT's dtype and the division runs in that dtype too (the reference
+        casts the encoder to bfloat16 before it quantises, eval_combo.py:351-352), then
+        q = clamp(rint(w / scale), -128, 127): the extreme weight of a channel lands on +-127.5,
+        i.e. on 127 (clamped from 128) or -128.  Not checked against torchao itself, which is
+        not installable here.
+    Either way the kernels only see int8 codes and an fp32 scale per channel."""
+    w = weight.detach()
+    if convention == "absmax127":
+        w = w.to(torch.float32)
+        scale = w.abs().amax(dim=1).clamp_min(1e-5) / 127.0
+        q = torch.round(w / scale[:, None]).clamp_(-127, 127).to(torch.int8)
+    elif convention == "torchao":
+        if not w.is_floating_point():
+            raise ValueError("the weight must be a floating-point tensor")
+        absmax = torch.maximum(w.amax(dim=1).clamp_min(0), (-w.amin(dim=1)).clamp_min(0))
+        scale = (absmax / 127.5).clamp(min=torch.finfo(torch.float32).eps).to(w.dtype)
+        q = torch.round(w / scale[:, None]).clamp_(-128, 127).to(torch.int8)
+    else:
+        raise ValueError(f"weight convention must be one of {WEIGHT_CONVENTIONS}, got {convention!r}")
+    return q.contiguous(), scale.to(torch.float32).contiguous()
 
 
 class Int8LinearBase(nn.Module):
@@ -42,7 +67,9 @@ class Int8LinearBase(nn.Module):
 
     Scales and the fp32 bias are registered as int32 bit patterns so that a
     later `model.to(torch.bfloat16)` (which casts every floating-point buffer)
-    cannot round them; they are viewed back as fp32 at call time."""
+    cannot round them; they are viewed back as fp32 at call time.  The bias has
+    this one home: `bias` is a read-only fp32 view of it, and a state dict that
+    carries a float `bias` entry (an nn.Linear's) is folded into it on load."""
 
     supports_row_scatter = True  # linear_fused accepts dst_row
 
@@ -53,11 +80,9 @@ class Int8LinearBase(nn.Module):
         self.out_features = out_features
         self.register_buffer("sw_bits", sw.to(torch.float32).contiguous().view(torch.int32))
         if bias is not None:
-            self.bias = nn.Parameter(bias.detach().clone(), requires_grad=False)
             self.register_buffer(
                 "bias_bits", bias.detach().to(torch.float32).contiguous().view(torch.int32))
         else:
-            self.bias = None
             self.bias_bits = None
 
     @property
@@ -69,6 +94,19 @@ class Int8LinearBase(nn.Module):
         return None if self.bias_bits is None else self.bias_bits.view(torch.float32)
 
     @property
+    def bias(self) -> Optional[torch.Tensor]:
+        return self.bias_f32
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        key = prefix + "bias"
+        if key in state_dict:
+            value = state_dict.pop(key)
+            if self.bias_bits is not None and prefix + "bias_bits" not in state_dict:
+                state_dict[prefix + "bias_bits"] = (
+                    value.detach().to(torch.float32).contiguous().view(torch.int32))
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
+    @property
     def weight(self) -> torch.Tensor:
         return self.wq.to(torch.float32) * self.sw[:, None]
 
@@ -77,13 +115,15 @@ class Int8LinearBase(nn.Module):
         raise NotImplementedError
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """The kernels compute on bf16 rows; any other floating input is cast on the way in and
+        the result cast back, so the module keeps its input's dtype as nn.Linear does."""
         lead = x.shape[:-1]
         x2 = x.reshape(-1, self.in_features)
         if x2.dtype != torch.bfloat16:
             x2 = x2.to(torch.bfloat16)
         xq, sx = ops.quant_rowwise(x2)
         y = self.linear_fused(xq, sx, EPILOGUE_NONE)
-        return y.reshape(*lead, self.out_features)
+        return y.reshape(*lead, self.out_features).to(x.dtype)
 
 
 class Int8DynamicLinear(Int8LinearBase):
@@ -97,8 +137,8 @@ class Int8DynamicLinear(Int8LinearBase):
         self._wq_kb64_key = None
 
     @classmethod
-    def from_float(cls, linear: nn.Linear) -> "Int8DynamicLinear":
-        wq, sw = quantize_weight_per_channel(linear.weight)
+    def from_float(cls, linear: nn.Linear, weight_convention: str = "absmax127") -> "Int8DynamicLinear":
+        wq, sw = quantize_weight_per_channel(linear.weight, weight_convention)
         return cls(linear.in_features, linear.out_features, wq, sw, linear.bias)
 
     def linear_fused(self, xq: torch.Tensor, sx: torch.Tensor, epilogue: int,
@@ -121,11 +161,17 @@ class Int8DynamicLinear(Int8LinearBase):
 
 
 def apply_dynamic_quant(model: nn.Module,
-                        filter_fn: Optional[Callable[[nn.Module, str], bool]] = None) -> None:
-    """Swap every nn.Linear under `model` for Int8DynamicLinear, in place."""
+                        filter_fn: Optional[Callable[[nn.Module, str], bool]] = None,
+                        weight_convention: str = "absmax127") -> None:
+    """Swap every nn.Linear under `model` for Int8DynamicLinear, in place.
+    `weight_convention` picks the per-channel weight quantiser (quantize_weight_per_channel):
+    "torchao" reproduces the codes and scales torchao's own swap would hold."""
+    if weight_convention not in WEIGHT_CONVENTIONS:
+        raise ValueError(f"weight convention must be one of {WEIGHT_CONVENTIONS}, got {weight_convention!r}")
     if filter_fn is None:
         filter_fn = lambda mod, fqn: isinstance(mod, nn.Linear)
     else:
         user = filter_fn
         filter_fn = lambda mod, fqn: isinstance(mod, nn.Linear) and user(mod, fqn)
-    replace_with_custom_fn_if_matches_filter(model, Int8DynamicLinear.from_float, filter_fn)
+    make = lambda linear: Int8DynamicLinear.from_float(linear, weight_convention)
+    replace_with_custom_fn_if_matches_filter(model, make, filter_fn)

@@ -86,7 +86,7 @@ def test_argument_validation_without_gpu():
     rc = lib.samfast_attn_relpos_fwd(p, p, p, p, p, p, 1, 1, 20, 20, 64, *([64] * 12), 0, 0.125, None)
     assert rc == -2 and b"neither" in lib.samfast_last_error()
     rc = lib.samfast_attn_relpos_fwd(p, p, p, p, p, p, 1, 1, 14, 14, 64, *([64] * 12), 1, 0.125, None)
-    assert rc == -2  # fp16 not built
+    assert rc == -2  # any element type other than SAMFAST_BF16
 
 
 def test_ops_refuse_cpu_tensors():
@@ -199,3 +199,80 @@ def test_checkpoint_with_reference_key_names_loads(tmp_path):
     q = sam.image_encoder.blocks[3].mlp.lin1
     assert isinstance(q, Int8DynamicLinear)
     assert (q.weight - w).abs().max() <= q.sw.max() * 0.5001
+
+
+def test_attention_wrappers_reject_mismatched_shapes_before_any_launch():
+    """The library is only told the grid; it would walk gh*gw tokens of every (batch, head) slice
+    whatever the tensors hold.  The wrappers therefore pin every shape on the host - these raise
+    on CPU tensors, i.e. before the device check and before anything could be launched."""
+    from samfast_amd import flash_4, ops
+    bf = torch.bfloat16
+    q = torch.zeros(1, 2, 2048, 64, dtype=bf)
+    tabs = torch.zeros(127, 64, dtype=bf)
+    with pytest.raises(RuntimeError, match="must be"):            # 2048 tokens on a 64x64 grid
+        ops.attn_relpos(q, q, q, tabs, tabs, (64, 64))
+    q4 = torch.zeros(1, 2, 4096, 64, dtype=bf)
+    with pytest.raises(RuntimeError, match="shape of q"):
+        ops.attn_relpos(q4, q4[:, :, :2048], q4, tabs, tabs, (64, 64))
+    with pytest.raises(RuntimeError, match="dtype of q"):
+        ops.attn_relpos(q4, q4.float(), q4, tabs, tabs, (64, 64))
+    with pytest.raises(RuntimeError, match="out must"):
+        ops.attn_relpos(q4, q4, q4, tabs, tabs, (64, 64), out=torch.zeros(1, 2, 2048, 64, dtype=bf))
+    rel_h = torch.zeros(1, 2, 2048, 64, dtype=bf)
+    with pytest.raises(RuntimeError, match="must be"):            # bias says 64x64 keys, q has 2048 tokens
+        ops.attn_relpos_bias(q, q, q, rel_h, rel_h)
+    with pytest.raises(RuntimeError, match="bias factors"):       # bias rows do not match q's tokens
+        ops.attn_relpos_bias(q4, q4, q4, rel_h, torch.zeros(1, 2, 4096, 64, dtype=bf))
+    with pytest.raises(RuntimeError, match="must be"):
+        ops.attn_relpos_windowed(q, q, q, torch.zeros(27, 64, dtype=bf), torch.zeros(27, 64, dtype=bf),
+                                 torch.zeros(2, 64, dtype=bf), torch.zeros(2, 64, dtype=bf), (64, 64), 14, 0.125)
+    # the registered operator derives the key grid from the token count: 64-wide rows only
+    with pytest.raises(RuntimeError, match="64-wide key grid"):
+        flash_4._custom_flash_aligned_gpu(q[:, :, :2000], q[:, :, :2000], q[:, :, :2000],
+                                          torch.zeros(1, 2, 2000, 128, dtype=bf), 0.125)
+    # a consistent call gets as far as the device check
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.attn_relpos(q4, q4, q4, tabs, tabs, (64, 64))
+
+
+def test_weight_quantiser_conventions_closed_form():
+    """The default per-channel convention (absmax / 127, clamp +-127) and torchao's
+    (absmax / 127.5 clamped at float32 eps, clamp -128..127, arithmetic in the weight's dtype),
+    on values whose quotients are exact."""
+    from samfast_amd.quant import quantize_weight_per_channel
+    w = torch.tensor([[127.0, -63.5, 1.0, 0.0], [-255.0, 255.0, 2.0, -1.0], [0.0, 0.0, 0.0, 0.0]])
+    q, s = quantize_weight_per_channel(w)
+    assert torch.equal(s, torch.tensor([1.0, 255.0 / 127.0, 1e-5 / 127.0]))
+    assert q.tolist() == [[127, -64, 1, 0], [-127, 127, 1, 0], [0, 0, 0, 0]]   # -63.5 -> -64: half to even
+    q, s = quantize_weight_per_channel(w, "torchao")
+    eps = torch.finfo(torch.float32).eps
+    assert torch.equal(s, torch.tensor([127.0 / 127.5, 2.0, eps]))
+    # row 1: +-255 / 2 = +-127.5 -> +-128 (half to even) -> clamped to 127 on the positive side only
+    assert q[1].tolist() == [-128, 127, 1, 0]
+    assert q[0].tolist() == [127, -64, 1, 0] and q[2].tolist() == [0, 0, 0, 0]   # 127.5 -> 128 -> 127; -63.75 -> -64
+    # bf16 weights: the scale is rounded to bf16 and the division runs in bf16, as torch would
+    wb = torch.tensor([[3.0, -1.0, 0.5, 0.25]], dtype=torch.bfloat16)
+    q, s = quantize_weight_per_channel(wb, "torchao")
+    sb = (torch.tensor(3.0) / 127.5).to(torch.bfloat16)
+    assert s.dtype == torch.float32 and torch.equal(s, sb.float()[None])
+    assert torch.equal(q, torch.round(wb / sb).clamp(-128, 127).to(torch.int8))
+    with pytest.raises(ValueError):
+        quantize_weight_per_channel(w, "other")
+
+
+def test_int8_linear_keeps_one_bias():
+    """The fp32 bias lives in one buffer; `bias` is a view of it, and loading a float `bias`
+    entry (what an nn.Linear state dict carries) lands in that buffer."""
+    from samfast_amd import Int8DynamicLinear
+    lin = nn.Linear(64, 16)
+    q = Int8DynamicLinear.from_float(lin, "torchao")
+    assert {k for k in q.state_dict()} == {"sw_bits", "bias_bits", "wq"}
+    assert torch.equal(q.bias, lin.bias.detach()) and q.bias.data_ptr() == q.bias_bits.data_ptr()
+    sd = q.state_dict()
+    del sd["bias_bits"]
+    sd["bias"] = torch.full((16,), 0.25, dtype=torch.bfloat16)
+    q.load_state_dict(sd)
+    assert torch.equal(q.bias_f32, torch.full((16,), 0.25))
+    q = q.to(torch.bfloat16)
+    assert q.bias.dtype == torch.float32
+    assert Int8DynamicLinear.from_float(nn.Linear(64, 16, bias=False)).bias is None

@@ -213,3 +213,102 @@ def test_derived_weight_copies_follow_load_state_dict():
         out = a(x)
     # stale copies would give an unrelated output; the neck convolutions are not run-to-run exact
     assert _cos(out, ref_b) >= 0.9995
+
+
+# ---- the ViT-H configurations at their full depth ------------------------------------------
+
+def _vit_h_state(seed=0):
+    from samfast_amd.build_sam import build_image_encoder
+    from samfast_amd.synthetic import init_encoder_weights
+    enc = build_image_encoder("vit_h")
+    sd = {k: v.clone() for k, v in init_encoder_weights(enc, seed=seed).items()}
+    return enc, sd
+
+
+def _trunk_input(enc, images):
+    """Patch embedding + position embedding (PyTorch-ROCm library GEMM), i.e. what block 0 receives."""
+    x = enc.patch_embed(images)
+    return x + enc.pos_embed if enc.pos_embed is not None else x
+
+
+def _run_blocks(enc, x):
+    for blk in enc.blocks:
+        x = blk(x)
+    return x
+
+
+def test_vit_h_all_32_blocks_vs_oracle():
+    """The ViT-H encoder at its full depth (32 blocks, 4 global), batch 2, seeded weights and images:
+    (a) attention kernels + int8 linears against the oracle that quantises the same way;
+    (b) attention kernels + bf16 nn.Linear against the float oracle.
+    Bar: cosine >= 0.999 per image, outputs finite."""
+    from samfast_amd import apply_dynamic_quant
+    enc, sd = _vit_h_state()
+    from samfast_amd.synthetic import make_images
+    x = make_images(2, seed=1).to(torch.bfloat16)
+    sd_r, xf = _rounded(sd), x.float()
+    lin = lambda a, w, b: oq.dynamic_int8_linear(a, w, b).float()
+    with torch.no_grad():
+        print("vit_h depth 32: float oracle ...", flush=True)
+        ref_f = oe.encoder_forward(sd_r, xf, oe.VIT_H, use_sdpa=True)
+        print("vit_h depth 32: quantised oracle ...", flush=True)
+        ref_q = oe.encoder_forward(sd_r, xf, oe.VIT_H, linear=lin, use_sdpa=True)
+        enc = enc.eval().to(torch.bfloat16).cuda()
+        out_f = enc(x.cuda()).float().cpu()
+        apply_dynamic_quant(enc)
+        assert all(b._int8_fused_ok(torch.empty(2, 64, 64, 1280, dtype=torch.bfloat16, device="cuda"))
+                   for b in enc.blocks)
+        out_q = enc(x.cuda()).float().cpu()
+    cf, cq, cqf = _cos(out_f, ref_f), _cos(out_q, ref_q), _cos(out_q, ref_f)
+    print(f"vit_h depth 32 bs2: bf16 linears vs float oracle {cf:.6f}; int8 vs quantised oracle {cq:.6f}; "
+          f"int8 vs float oracle {cqf:.6f}", flush=True)
+    assert torch.isfinite(out_f).all() and torch.isfinite(out_q).all()
+    assert cf >= COSINE_MIN and cq >= COSINE_MIN
+    assert cqf >= 0.995  # quantisation noise itself, against the unquantised model
+
+
+def test_vit_h_batch_16_blocks_bitwise_equal_batch_2_runs():
+    """Images are independent and every kernel here is deterministic, so the 32 blocks applied to a
+    batch of 16 must give, image by image, the very bits they give on batches of 2 - whatever tile,
+    workgroup or wave count the larger launch picks.  (The patch embedding in front is a library
+    GEMM whose algorithm may change with the batch: both runs start from the same embedded tokens.)"""
+    from samfast_amd import apply_dynamic_quant
+    from samfast_amd.synthetic import make_images
+    enc, _ = _vit_h_state()
+    enc = enc.eval().to(torch.bfloat16).cuda()
+    apply_dynamic_quant(enc)
+    with torch.no_grad():
+        x0 = _trunk_input(enc, make_images(16, seed=1).to(torch.bfloat16).cuda())
+        full = _run_blocks(enc, x0.clone())
+        torch.cuda.synchronize()
+        assert torch.isfinite(full.float()).all()
+        for i in (0, 6, 14):
+            part = _run_blocks(enc, x0[i:i + 2].clone())
+            assert torch.equal(part.view(torch.int16), full[i:i + 2].view(torch.int16)), i
+        out = enc.neck(full.permute(0, 3, 1, 2))
+    assert out.shape == (16, 256, 64, 64) and torch.isfinite(out.float()).all()
+
+
+def test_vit_h_batch_32_sparse_mlp_bitwise_equals_dense_kernels_on_pruned_weights():
+    """The int8 + 2:4 configuration at its real batch (32 images, all 32 blocks): the sparse matrix
+    cores on the packed lin1 / lin2 weights must reproduce, bit for bit, the dense int8 kernels run on
+    the same magnitude-pruned weights (integer accumulators are exact, the epilogues are shared)."""
+    from samfast_amd import apply_dynamic_quant, apply_fake_sparsity, apply_sparse
+    from samfast_amd.sparse import Int8Sparse24Linear, mlp_only
+    from samfast_amd.synthetic import make_images
+    a, sd = _vit_h_state()
+    b, _ = _vit_h_state()
+    a = a.eval().to(torch.bfloat16).cuda()
+    b = b.eval().to(torch.bfloat16).cuda()
+    apply_sparse(a, mlp_only)
+    apply_dynamic_quant(a)
+    apply_fake_sparsity(b, mlp_only)
+    apply_dynamic_quant(b)
+    assert isinstance(a.blocks[5].mlp.lin2, Int8Sparse24Linear) and not isinstance(b.blocks[5].mlp.lin2, Int8Sparse24Linear)
+    with torch.no_grad():
+        x0 = _trunk_input(a, make_images(32, seed=1).to(torch.bfloat16).cuda())
+        ya = _run_blocks(a, x0.clone())
+        yb = _run_blocks(b, x0.clone())
+    torch.cuda.synchronize()
+    assert torch.isfinite(ya.float()).all()
+    assert torch.equal(ya.view(torch.int16), yb.view(torch.int16))

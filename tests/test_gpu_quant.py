@@ -360,3 +360,52 @@ def test_quantiser_exact_ties_round_to_even():
     expect = np.array([int(np.rint(k + 0.5)) for k in range(64)])     # numpy rint: half to even
     assert sx_ref[0] == np.float32(1.0) and np.array_equal(got, expect) and got[0] == 0 and got[1] == 2 and got[2] == 2
     assert np.array_equal(xq[0, 65:129].cpu().numpy(), -expect)
+
+
+def test_nan_in_a_row_reaches_the_linear_output():
+    """A NaN anywhere in a row gives that row a NaN scale (plain and LayerNorm form), so the Linear
+    that reads it returns NaN for that row and for no other - as a float Linear would.  The oracle's
+    maximum propagates the NaN the same way."""
+    from samfast_amd import ops
+    x, w, b = linear_inputs(40, 1280, 256, seed=3)
+    x[7, 100] = float("nan")
+    x[21, 1279] = float("nan")
+    _, s_ref = orq.quantize_rows_absmax(x)
+    bad = np.isnan(s_ref)
+    assert bad.sum() == 2 and bad[7] and bad[21]
+    wq, sw = ops.quant_rowwise(w.cuda())
+    gamma, beta = torch.ones(1280, dtype=torch.bfloat16).cuda(), torch.zeros(1280, dtype=torch.bfloat16).cuda()
+    for xq, sx in (ops.quant_rowwise(x.cuda()), ops.layernorm_quant(x.cuda(), gamma, beta, 1e-6)):
+        assert np.array_equal(np.isnan(sx.cpu().numpy()), bad)
+        y = ops.gemm_i8_scale_bias(xq, sx, wq, sw, b.float().cuda()).float().cpu()
+        rows = torch.isnan(y).all(dim=1).numpy()
+        assert np.array_equal(rows, bad) and torch.isfinite(y[~torch.from_numpy(bad)]).all()
+    # finite rows are untouched by their neighbours' NaNs
+    xq, sx = ops.quant_rowwise(x.cuda())
+    q_ref, _ = orq.quantize_rows_absmax(x)
+    assert np.array_equal(xq.cpu().numpy()[~bad], q_ref[~bad]) and np.array_equal(sx.cpu().numpy()[~bad], s_ref[~bad])
+
+
+@pytest.mark.parametrize("K,mean,std", [(1280, 0.0, 1.0), (1280, 40.0, 0.25), (768, -3.0, 5.0), (5120, 10.0, 0.05)])
+def test_layernorm_quant_statistics_against_float64(K, mean, std):
+    """The LayerNorm + quantiser kernel against LayerNorm evaluated in float64 on the same bf16
+    inputs, including rows whose mean dwarfs their spread (where a one-pass variance would cancel).
+    Dequantised codes must reproduce the float64 result to half a quantisation step plus one bf16
+    rounding of the normalised value (2^-8 relative) plus the fp32 statistics' error (1e-4);
+    the scale must be the float64 absmax / 127 to the same bf16 rounding."""
+    from samfast_amd import ops
+    g = torch.Generator().manual_seed(K)
+    x = (torch.randn(64, K, generator=g) * std + mean).to(torch.bfloat16)
+    gamma = (1 + 0.1 * torch.randn(K, generator=g)).to(torch.bfloat16)
+    beta = (0.1 * torch.randn(K, generator=g)).to(torch.bfloat16)
+    x64, g64, b64 = x.double(), gamma.double(), beta.double()
+    mu = x64.mean(dim=1, keepdim=True)
+    var = ((x64 - mu) ** 2).mean(dim=1, keepdim=True)
+    y64 = (x64 - mu) / torch.sqrt(var + 1e-6) * g64 + b64
+    q, s = ops.layernorm_quant(x.cuda(), gamma.cuda(), beta.cuda(), 1e-6)
+    q, s = q.cpu().double(), s.cpu().double()
+    amax = y64.abs().amax(dim=1)
+    assert ((s * 127 - amax).abs() <= amax * (2.0 ** -8 + 1e-4)).all()
+    err = (q * s[:, None] - y64).abs()
+    bound = 0.5 * s[:, None] + y64.abs() * (2.0 ** -8 + 1e-4) + 1e-4
+    assert (err <= bound).all(), (err - bound).max().item()

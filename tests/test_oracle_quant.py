@@ -48,7 +48,7 @@ def test_quantiser_invariants():
     assert np.array_equal(q3[keep], q[keep])
 
 
-@pytest.mark.parametrize("M,N,K", [(3, 8, 8), (17, 24, 64), (130, 264, 1280)])
+@pytest.mark.parametrize("M,N,K", [(3, 8, 8), (17, 24, 64), (130, 264, 1280), (256, 1280, 1280)])
 def test_int8_gemm_three_ways(M, N, K):
     g = torch.Generator().manual_seed(M + N + K)
     a = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).numpy()
@@ -56,6 +56,9 @@ def test_int8_gemm_three_ways(M, N, K):
     ref64 = orq.int8_gemm_i64(a, b)
     got = orq.int8_gemm_i32(a, b)
     assert got.dtype == np.int32 and np.array_equal(got.astype(np.int64), ref64)
+    if M > 16 and K % 8 == 0 and N % 8 == 0:  # the library routine the reference's quantised Linear calls
+        lib = torch._int_mm(torch.from_numpy(a), torch.from_numpy(b).t())
+        assert np.array_equal(lib.numpy(), got)
     # brute force on a corner
     for (i, j) in [(0, 0), (M - 1, N - 1)]:
         assert ref64[i, j] == sum(int(a[i, t]) * int(b[j, t]) for t in range(K))
