@@ -7,11 +7,16 @@ all four Linears of every block on the dynamic-int8 HIP kernels), inputs and
 weights resident in HBM before the timed region.
 
 Prints ONE JSON line: images/s plus
-  roofline      the dominant kernel (by time inside a step) against its bound,
-                from per-launch event timings of an instrumented step;
-  kernels       the same figures for every hand-written kernel in the step;
-  gpu_baseline  the same encoder through PyTorch-ROCm bf16 SDPA + bf16 Linear;
-  cpu_baseline  the CPU oracle (the reference's eager route) on one image.
+  roofline       the dominant kernel (by time inside a step) against its bound,
+                 from per-launch event timings of an instrumented step;
+  kernels        the same figures for every hand-written kernel in the step;
+  gpu_baseline   the same encoder through PyTorch-ROCm bf16 SDPA + bf16 Linear;
+  other_configs  the two other encoder configurations of the benchmark, measured the same way in the
+                 same process: ViT-H batch 32 with 2:4-sparse MLP linears, and ViT-B batch 1 (eager
+                 launches and replayed as one HIP graph); --main-only leaves them out;
+  mfma_ceiling   what a loop of nothing but matrix instructions sustains on this GPU, on constant and
+                 on random operands (--no-mfma-ceiling leaves it out);
+  cpu_baseline   the CPU oracle (the reference's eager route) on one image.
 """
 
 import argparse
@@ -31,11 +36,13 @@ PEAK = {"op": ("mfma", 5.0e15, "TOP/s"),       # int8 dense MFMA
 
 # Bytes per launch that cross the L2 <-> fabric boundary (average over the launches of one
 # encoder step), from the two `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this
-# script summarised in profiles/bench_vit_h_bs16_pmc_traffic.txt, each counter scaled by what
-# it reads for the 1 GiB --calibration-copy dispatch (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
-# Valid for the default workload (vit_h, batch 16, dense int8 linears) only.
-TRAFFIC = {"gemm_i8_kernel": 1.0587e9, "attn_window": 6.728e8, "attn_global": 7.740e8,
-           "quant_rowwise": 6.304e8, "layernorm_quant": 2.543e8}
+# script summarised in TRAFFIC_SOURCE, each counter scaled by what it reads for the 1 GiB
+# --calibration-copy dispatch (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Counters cannot be read
+# from inside a timed run, so the figure is a recorded one: it is reported only for the default
+# workload (vit_h, batch 16, dense int8 linears) and only while the kernel's source file still
+# has the hash it had when the counters were taken (otherwise `traffic` is null).
+TRAFFIC_SOURCE = "profiles/bench_vit_h_bs16_pmc_traffic.txt"
+TRAFFIC = {"gemm_i8_kernel": (1.0587e9, "gemm_i8.hip", "e6c828909dfa3b6e")}
 
 
 def parse():
@@ -47,6 +54,11 @@ def parse():
     p.add_argument("--batch", type=int, default=16)
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-gpu-baseline", action="store_true")
+    p.add_argument("--main-only", action="store_true",
+                   help="measure only the workload named by --model / --batch (no other_configs object)")
+    p.add_argument("--no-mfma-ceiling", action="store_true", help="skip the matrix-instruction-only loops")
+    p.add_argument("--mfma-ceiling", action="store_true",
+                   help="run ONLY the matrix-instruction-only loops and print their JSON object")
     p.add_argument("--bf16-linears", action="store_true", help="keep nn.Linear (attention kernels only)")
     p.add_argument("--sparse-mlp", action="store_true",
                    help="lin1 / lin2 magnitude-pruned 2:4 on the sparse int8 matrix cores (the int8 + 2:4 "
@@ -155,50 +167,95 @@ def library_yardsticks(batch, heads, hd, width):
     return res
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (no collectives exist on this path); "
-              "use --gpus 1", file=sys.stderr)
-        sys.exit(2)
+def source_sha16(name):
+    import hashlib
+    path = ROOT / "segment-anything-fast_amd" / "csrc" / name
+    return hashlib.sha256(path.read_bytes()).hexdigest()[:16] if path.exists() else None
 
+
+def mfma_ceiling():
+    """Loops of nothing but matrix instructions (operands in registers, no memory traffic), on
+    operands that are all zero, small constants, and random like a GEMM's / attention's: the
+    rate this GPU's matrix pipe sustains under its power limit, in POP/s (int8) and PFLOP/s (bf16)."""
+    import ctypes
+    import torch
+    from samfast_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    out = torch.zeros(1024, dtype=torch.int32, device=dev)
+    g = torch.Generator(device="cuda").manual_seed(7)
+    n8 = 8 * 256 * 16   # bytes of one operand buffer
+    operands = {
+        0: {"zeros": torch.zeros(n8, dtype=torch.int8, device=dev),
+            "small_ints": torch.randint(0, 3, (n8,), generator=g, dtype=torch.int8, device=dev),
+            "random_int8": torch.randint(-127, 128, (n8,), generator=g, dtype=torch.int8, device=dev)},
+        1: {"zeros": torch.zeros(n8 // 2, dtype=torch.bfloat16, device=dev),
+            "ones": torch.ones(n8 // 2, dtype=torch.bfloat16, device=dev),
+            "random_normal": torch.randn(n8 // 2, generator=g, device=dev).to(torch.bfloat16)},
+    }
+    res = {"what": "8 independent MFMAs per round and wavefront, operands in registers, 512 workgroups of "
+                   "4 wavefronts (2 wavefronts per SIMD on 256 CUs), ~40 ms per launch, events on the launch stream",
+           "int8_v_mfma_i32_32x32x32_i8": {"unit": "POP/s", "published_peak": 5.0},
+           "bf16_v_mfma_f32_32x32x16_bf16": {"unit": "PFLOP/s", "published_peak": 2.5}}
+    stream = torch.cuda.current_stream().cuda_stream
+    for instr, key, iters in ((0, "int8_v_mfma_i32_32x32x32_i8", 120000), (1, "bf16_v_mfma_f32_32x32x16_bf16", 100000)):
+        for name, buf in operands[instr].items():
+            ops = ctypes.c_int64(0)
+            launch = lambda: _lib.check(lib.samfast_bench_mfma_ceiling(
+                instr, buf.data_ptr(), 512, iters, ctypes.byref(ops), out.data_ptr(), stream), "bench_mfma_ceiling")
+            launch()
+            torch.cuda.synchronize()
+            best = 0.0
+            for _ in range(3):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                launch()
+                e1.record()
+                torch.cuda.synchronize()
+                best = max(best, ops.value / (e0.elapsed_time(e1) * 1e-3) / 1e15)
+            res[key][name] = round(best, 3)
+    return res
+
+
+def run_config(model, batch, steps, warmup, sparse_mlp=False, bf16_linears=False, graph=False,
+               gpu_baseline=True, calibration_copy=False, yardsticks=False, also_graph=False):
+    """Build the encoder, time `steps` forwards after `warmup`, run one instrumented forward for the
+    per-kernel figures and (optionally) the PyTorch-ROCm eager baseline on the same weights."""
     import torch
     from samfast_amd import apply_dynamic_quant, apply_sparse, flash_4, ops
     from samfast_amd.sparse import mlp_only
     from samfast_amd.build_sam import build_image_encoder
     from samfast_amd.synthetic import init_encoder_weights, make_images
-
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
 
-    enc = build_image_encoder(args.model)
+    enc = build_image_encoder(model)
     sd_fp32 = {k: v.clone() for k, v in init_encoder_weights(enc, seed=0).items()}
     enc = enc.eval().to(torch.bfloat16).to(dev)
-    if args.sparse_mlp:
+    if sparse_mlp:
         apply_sparse(enc, mlp_only)
-    if not args.bf16_linears:
+    if not bf16_linears:
         apply_dynamic_quant(enc)
-    images = make_images(args.batch, seed=1).to(torch.bfloat16).to(dev)
+    images = make_images(batch, seed=1).to(torch.bfloat16).to(dev)
 
-    if args.calibration_copy:
+    if calibration_copy:
         src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
         dst = torch.empty_like(src)
         dst.copy_(src)  # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
 
+    extra = {}
     with torch.no_grad():
         step = lambda: enc(images)
-        if args.graph:
+        if graph or also_graph:
             from samfast_amd.graphs import GraphedEncoder
             graphed = GraphedEncoder(enc, images)
-            timed = lambda: graphed(images)
-        else:
-            timed = step
-        sec = time_steps(timed, args.steps, args.warmup)
+        timed = (lambda: graphed(images)) if graph else step
+        sec = time_steps(timed, steps, warmup)
+        if also_graph and not graph:
+            gsec = time_steps(lambda: graphed(images), steps, warmup)
+            extra["hip_graph_replay"] = {"value": round(batch / gsec, 3), "unit": "images/s",
+                                         "ms_per_step": round(gsec * 1e3, 3)}
         out = step()
         finite = bool(torch.isfinite(out.float()).all())
 
@@ -220,40 +277,44 @@ def main():
     families = kernel_table(fam)
     dominant = max(families, key=lambda n: families[n]["ms_total"])
     dk = families[dominant]
+    traffic, traffic_note = None, "not measured for this workload"
+    if (model, batch, sparse_mlp, bf16_linears) == ("vit_h", 16, False, False) and dominant in TRAFFIC:
+        value, src_name, sha = TRAFFIC[dominant]
+        if source_sha16(src_name) == sha:
+            traffic, traffic_note = value, f"rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in {TRAFFIC_SOURCE}"
+        else:
+            traffic_note = (f"{src_name} changed since the counters in {TRAFFIC_SOURCE} were taken "
+                            f"(then {value / 1e6:.0f} MB per launch)")
     roofline = {"kernel": dominant, "bound": dk["bound"], "achieved": dk["achieved"],
                 "peak": dk["peak"], "unit": dk["unit"], "frac": dk["frac"],
-                "traffic": TRAFFIC.get(dominant)
-                if (args.model, args.batch, args.sparse_mlp) == ("vit_h", 16, False) else None,
+                "traffic": traffic, "traffic_source": traffic_note,
                 "avg_us": dk["avg_us"], "launches_per_step": dk["launches"],
                 "ms_per_step": dk["ms_total"]}
 
     result = {
-        "metric": ("images/s ViT-H encoder bs16 1024^2" if (args.model, args.batch) == ("vit_h", 16)
-                   else f"images/s {args.model} encoder bs{args.batch} 1024^2")
-        + (" (2:4 sparse MLP)" if args.sparse_mlp else ""),
-        "value": round(args.batch / sec, 3), "unit": "images/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 3),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": ("bf16" if args.bf16_linears and not args.sparse_mlp else
+        "value": round(batch / sec, 3), "unit": "images/s", "ms_per_step": round(sec * 1e3, 3),
+        "steps": steps, "warmup": warmup,
+        "dtype": ("bf16" if bf16_linears and not sparse_mlp else
                   "bf16 attention + int8 linears (int32 accumulate)"
-                  + (", lin1/lin2 2:4 sparse" if args.sparse_mlp else "")),
-        "data": "synthetic (seeded uniform images, random-init weights)",
-        "config": {"workload": f"SAM {args.model} image encoder forward, batch {args.batch}, "
-                               "1024x1024, rel-pos attention + dynamic int8 linears"
-                               + (" (lin1 / lin2 pruned 2:4, sparse int8 MFMA)" if args.sparse_mlp else ""),
-                   "batch": args.batch, "image": 1024},
-        "hip_graph": bool(args.graph),
+                  + (", lin1/lin2 2:4 sparse" if sparse_mlp else "")),
+        "config": {"workload": f"SAM {model} image encoder forward, batch {batch}, "
+                               "1024x1024, rel-pos attention + "
+                               + ("bf16 linears" if bf16_linears and not sparse_mlp else "dynamic int8 linears")
+                               + (" (lin1 / lin2 pruned 2:4, sparse int8 MFMA)" if sparse_mlp else ""),
+                   "batch": batch, "image": 1024},
+        "hip_graph": bool(graph),
         "output_finite": finite,
         "roofline": roofline,
         "kernels": kernels,
     }
+    result.update(extra)
 
-    if not args.no_gpu_baseline:
+    if gpu_baseline:
         # same weights, PyTorch-ROCm eager: bf16 nn.Linear + SDPA with a materialised bias
-        base = build_image_encoder(args.model)
+        base = build_image_encoder(model)
         base.load_state_dict(sd_fp32)
         base = base.eval().to(torch.bfloat16).to(dev)
-        if args.sparse_mlp:  # same pruned weights, dense bf16 kernels
+        if sparse_mlp:  # same pruned weights, dense bf16 kernels
             from samfast_amd import apply_fake_sparsity
             apply_fake_sparsity(base, mlp_only)
         flash_4.USE_CUSTOM_KERNEL = False
@@ -266,22 +327,96 @@ def main():
         finally:
             flash_4.USE_CUSTOM_KERNEL = True
         result["gpu_baseline"] = {"what": "same encoder, PyTorch-ROCm eager bf16 SDPA(attn_mask) + bf16 nn.Linear",
-                                  "value": round(args.batch / bsec, 3), "unit": "images/s",
+                                  "value": round(batch / bsec, 3), "unit": "images/s",
                                   "ms_per_step": round(bsec * 1e3, 3),
                                   "speedup": round(bsec / sec, 3),
                                   "min_cosine_vs_this_path": round(cos, 6)}
         del base, ref
-        torch.cuda.empty_cache()
 
-    if args.library_yardsticks:
+    if yardsticks:
         blk = enc.blocks[0].attn
         with torch.no_grad():
             result["library_yardsticks"] = library_yardsticks(
-                args.batch, blk.num_heads, blk.qkv.in_features // blk.num_heads, blk.qkv.in_features)
+                batch, blk.num_heads, blk.qkv.in_features // blk.num_heads, blk.qkv.in_features)
+    del enc, images, out
+    torch.cuda.empty_cache()
+    return result, sd_fp32
+
+
+def brief(r):
+    """What an other_configs entry keeps of a run_config result."""
+    keep = {k: r[k] for k in ("value", "unit", "ms_per_step", "steps", "warmup", "dtype", "output_finite")}
+    keep["workload"] = r["config"]["workload"]
+    rf = r["roofline"]
+    keep["dominant_kernel"] = {k: rf[k] for k in ("kernel", "bound", "achieved", "peak", "unit", "frac",
+                                                   "avg_us", "launches_per_step", "ms_per_step")}
+    keep["kernels"] = {n: {k: d[k] for k in ("launches", "ms_total", "achieved", "unit", "frac")}
+                       for n, d in r["kernels"].items()}
+    for k in ("gpu_baseline", "hip_graph_replay"):
+        if k in r:
+            keep[k] = r[k]
+    return keep
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives exist on this path); "
+              "use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from samfast_amd.synthetic import make_images
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(torch.device("cuda:0"))
+
+    if args.mfma_ceiling:
+        print(json.dumps({"mfma_ceiling": mfma_ceiling()}))
+        return
+
+    main_run, sd_fp32 = run_config(
+        args.model, args.batch, args.steps, args.warmup, sparse_mlp=args.sparse_mlp,
+        bf16_linears=args.bf16_linears, graph=args.graph, gpu_baseline=not args.no_gpu_baseline,
+        calibration_copy=args.calibration_copy, yardsticks=args.library_yardsticks)
+
+    result = {
+        "metric": ("images/s ViT-H encoder bs16 1024^2" if (args.model, args.batch) == ("vit_h", 16)
+                   else f"images/s {args.model} encoder bs{args.batch} 1024^2")
+        + (" (2:4 sparse MLP)" if args.sparse_mlp else ""),
+        "value": main_run["value"], "unit": "images/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_run["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": main_run["dtype"],
+        "data": "synthetic (seeded uniform images, random-init weights)",
+        "config": main_run["config"],
+    }
+    for k in ("hip_graph", "output_finite", "roofline", "kernels", "gpu_baseline", "library_yardsticks"):
+        if k in main_run:
+            result[k] = main_run[k]
+
+    default_workload = (args.model, args.batch, args.sparse_mlp, args.bf16_linears, args.graph) == \
+        ("vit_h", 16, False, False, False)
+    if default_workload and not args.main_only:
+        # the benchmark's two other encoder configurations, same protocol, fewer steps
+        others = {}
+        r, _ = run_config("vit_h", 32, max(3, args.steps // 2), 2, sparse_mlp=True,
+                          gpu_baseline=not args.no_gpu_baseline)
+        others["vit_h_bs32_int8_sparse24_mlp"] = brief(r)
+        r, _ = run_config("vit_b", 1, max(20, args.steps), 5, gpu_baseline=not args.no_gpu_baseline,
+                          also_graph=True)
+        others["vit_b_bs1_int8"] = brief(r)
+        result["other_configs"] = others
+
+    if not args.no_mfma_ceiling:
+        result["mfma_ceiling"] = mfma_ceiling()
 
     if not args.no_cpu_baseline:
         from oracle import image_encoder as oe
         cfg = {"vit_h": oe.VIT_H, "vit_l": oe.VIT_L, "vit_b": oe.VIT_B}[args.model]
+        # the host share of a one-GPU box is 16 cores whatever os.cpu_count() shows there
         cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
         torch.set_num_threads(cores)
         n_cpu = 3 if args.model == "vit_h" else 6  # about 10-15 s of host work
