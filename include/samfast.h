@@ -207,6 +207,30 @@ int samfast_gemm_i8_fused(
     const void* residual, int64_t ld_res, const int32_t* dst_row, int layout, void* stream);
 
 /*
+ * samfast_gemm_i8_fused (epilogues NONE / GELU / RESIDUAL, no row scatter) that also hands the
+ * NEXT Linear its quantised input: after y is written, each row of y - passed through LayerNorm
+ * first when ln_gamma / ln_beta (N values of type `dtype`) are given - is quantised per row exactly
+ * as samfast_quant_rowwise_i8 / samfast_layernorm_quant_i8 would quantise it, into yq (M, N) int8 in
+ * `yq_layout` and sy (M) fp32; codes and scales are bit-equal to those two calls on y.  Stands for
+ * what the compiler fuses around the reference's quantised Linears: lin1 + GELU + lin2's activation
+ * quantiser (modeling/common.py:25-26), proj + residual + norm2 + lin1's quantiser and lin2 +
+ * residual + the next block's norm1 + qkv's quantiser (modeling/image_encoder.py:167-183).
+ * Where the shape allows (K >= 256; GELU with N in {3072, 4096, 5120}, or RESIDUAL + LayerNorm with
+ * N in {768, 1024, 1280}) everything is ONE launch: the workgroup that completes a 128-row tile
+ * quantises its rows (no workgroup ever waits for another); other shapes run as two launches.
+ * `tile_counters`: device workspace of at least ceil(M / 128) int32, all zero on entry; the launch
+ * leaves it all zero again, so one buffer serves every call on a stream.  Calls that share a counter
+ * buffer must not overlap in time (use one buffer per stream).
+ */
+int samfast_gemm_i8_fused_quant(
+    const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
+    const float* bias, void* y, int64_t ldy,
+    int64_t M, int N, int K, int dtype, int epilogue,
+    const void* residual, int64_t ld_res, int layout,
+    const void* ln_gamma, const void* ln_beta, float ln_eps,
+    int8_t* yq, float* sy, int yq_layout, int32_t* tile_counters, void* stream);
+
+/*
  * 2:4-sparse weights for the sparse int8 matrix cores (v_smfmac_i32_32x32x64_i8).
  *
  * samfast_prune24_pack_i8: from a dense int8 weight wq (N, K) keep, in every aligned group

@@ -38,7 +38,18 @@
 // group when there are few (the column tiles of a row tile run side by side and share X).
 // Outputs larger than the last-level cache that carry no residual (qkv, lin1: read once by
 // the next kernel) are written with streaming stores.
-#include "samfast_internal.hpp"
+//
+// Quantiser of the output inside the GEMM (TAILN > 0).  The next Linear wants the rows this
+// GEMM produces quantised per row, (LayerNorm first where one sits between them,) and a row's
+// scale needs the whole row, which the tiles_n workgroups of a row tile produce between them.
+// Nobody waits for anybody: a workgroup stores its tile, makes the stores visible to the whole
+// device (release fence at agent scope) and adds one to the row tile's counter with a
+// device-scope atomic; the workgroup that reads tiles_n - 1 knows every other tile of these 128
+// rows is complete and visible, acquires, and runs the row quantiser (the code of
+// quant_rowwise.hip, one wavefront per row, rows double-buffered) over them, then puts the
+// counter back to zero for the next launch.  The other workgroup resident on the CU keeps the
+// matrix pipe busy meanwhile.
+#include "quant_row.hpp"
 #include <stdlib.h>
 #include <type_traits>
 
@@ -70,6 +81,14 @@ struct GemmArgs {
   const unsigned short* residual;  // EPI_RESIDUAL: (rows, N) bf16, row stride ld_res
   int64_t ld_res;
   const int32_t* dst_row;          // EPI_RESIDUAL: output row per GEMM row, -1 = drop; may be null
+  // quantiser of the output rows (kernels with TAILN > 0)
+  int32_t* tile_counters;          // one per row tile; zero before the launch and again after it
+  int8_t* yq;                      // codes of the (LayerNorm of the) output rows, layout yq_kb64
+  float* sy;                       // their scales
+  const unsigned short* ln_gamma;  // TAILLN: LayerNorm weight / bias (N bf16 values each)
+  const unsigned short* ln_beta;
+  float ln_eps;
+  int yq_kb64;
 };
 
 // Epilogue shared by the kernels: the lane owns 4 adjacent output columns of each of
@@ -296,19 +315,71 @@ SF_DEVICE void gemm_epilogue_staged(const GemmArgs& a, i32x16 (&acc)[2][4], unsi
   }
 }
 
+// The quantiser tail (see the file header).  Called by every thread of the workgroup after its
+// last output store; `flag` is one LDS word nobody else uses any more.
+template <int TAILN, bool TAILLN>
+SF_DEVICE void gemm_quant_tail(const GemmArgs& a, int m0, int tile_m, int tid, int* flag) {
+  constexpr int EPC = quant_epc_for(TAILN), NCH = quant_nch_for(TAILN);
+  using RQ = RowQuantizer<NCH, EPC, TAILLN>;
+  // every wavefront's stores have completed (vmcnt counts stores as well), then one thread
+  // releases them - the fence is cumulative over what the barrier ordered before it
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  __builtin_amdgcn_s_barrier();
+  if (tid == 0) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    *flag = __hip_atomic_fetch_add(a.tile_counters + tile_m, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (*flag != a.tiles_n - 1) return;  // uniform: somebody else will be the last
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+
+  QuantArgs q;
+  q.x = reinterpret_cast<const unsigned short*>(a.out);
+  q.ldx = a.ldo;
+  q.gamma = a.ln_gamma; q.beta = a.ln_beta; q.src_row = nullptr;
+  q.xq = a.yq; q.sx = a.sy; q.M = a.M; q.K = TAILN;
+  q.eps = a.ln_eps; q.inv_K = 1.0f / (float)TAILN; q.kb64 = a.yq_kb64;
+  constexpr int nchunk = TAILN / EPC;
+  const int lane = tid & 63, wave = tid >> 6;
+  typename RQ::in_t gw[NCH], bw[NCH];
+  if (TAILLN) RQ::load_affine(q.gamma, q.beta, nchunk, lane, gw, bw);
+  // wavefront w takes rows w, w + 4, ...; the loads of the next DEPTH - 1 rows are in flight while
+  // one row is worked on (a lone wavefront per SIMD has nobody else to hide their latency)
+  constexpr int DEPTH = NCH * RQ::W <= 12 ? 6 : 2;
+  typename RQ::in_t buf[DEPTH][NCH];
+  const int last = min(m0 + 128, a.M);
+  const int row0 = m0 + wave;
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (row0 + 4 * d < last) RQ::template load_row<false>(q.x + (int64_t)(row0 + 4 * d) * q.ldx, nchunk, lane, buf[d]);
+  for (int base = row0; base < last; base += 4 * DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int row = base + 4 * d;
+      if (row < last) {  // uniform over the wavefront
+        RQ::finish_row(q, row, nchunk, lane, buf[d], gw, bw);
+        const int next = row + 4 * DEPTH;
+        if (next < last) RQ::template load_row<false>(q.x + (int64_t)next * q.ldx, nchunk, lane, buf[d]);
+      }
+    }
+  }
+  if (tid == 0) a.tile_counters[tile_m] = 0;  // the next launch finds the counter at zero
+}
+
 // 16-byte chunk c of LDS row r lives at chunk position c ^ lds_swizzle(r).  With it the
 // operand reads (one chunk of 8 / 16 consecutive rows per LDS cycle) and the tile writes
 // (4 chunks of 2 / 4 consecutive rows per cycle) both touch every bank once, whether the
 // LDS cycles through 128 or 256 bytes.
 SF_DEVICE int lds_swizzle(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
 
-template <int EPI, int TM, bool GENERIC>
+template <int EPI, int TM, bool GENERIC, int TAILN = 0, bool TAILLN = false>
 __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArgs a) {
   constexpr int GBM = 64 * TM;
   constexpr int GSTAGE = (GBM + GBN) * GLD;
   constexpr int NST = GENERIC ? 2 : (TM == 4 ? 4 : 3);  // LDS stages
   constexpr bool STAGED = !GENERIC && TM == 2 && EPI != EPI_I32;  // epilogue through LDS
   static_assert(!STAGED || 128 * EP_STRIDE <= NST * GSTAGE, "output tile must fit in the operand stages");
+  static_assert(TAILN == 0 || STAGED, "the quantiser tail follows the staged epilogue");
   __shared__ __attribute__((aligned(16))) unsigned char lds[NST * GSTAGE + (STAGED ? EP_SCALE_BYTES + EP_ROWMAP_BYTES : 0)];
 
   const int tid = threadIdx.x;
@@ -570,13 +641,40 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
     gemm_epilogue_staged<EPI>(a, acc, lds, lds + NST * GSTAGE, m0, n0, wm, wn, lr, lh, tid);
   else
     gemm_epilogue<EPI, TM>(a, acc, m0, n0, wm, wn, lr, lh);
+  if constexpr (TAILN > 0)
+    gemm_quant_tail<TAILN, TAILLN>(a, m0, m0 / GBM, tid, reinterpret_cast<int*>(lds + NST * GSTAGE));
+}
+
+// the output quantiser a launch may carry (null = none)
+struct GemmTail {
+  int8_t* yq;
+  float* sy;
+  const void* gamma;  // non-null: LayerNorm before the quantiser
+  const void* beta;
+  float eps;
+  int yq_layout;
+  int32_t* counters;
+};
+
+// N for which the quantiser tail is built, per kind: plain after GELU (the MLP widths of
+// ViT-B / L / H), LayerNorm after a residual epilogue (their embedding widths)
+static bool tail_built(int epi, bool ln, int N) {
+  if (epi == EPI_GELU_BF16 && !ln) return N == 3072 || N == 4096 || N == 5120;
+  if (epi == EPI_RESIDUAL_BF16 && ln) return N == 768 || N == 1024 || N == 1280;
+  return false;
+}
+
+// whether gemm_common would run `tail` inside the GEMM for this call
+static bool tail_fusable(int epi, const GemmTail& t, int N, int K, const int32_t* dst_row) {
+  const char* force = getenv("SAMFAST_GEMM_TM");
+  return K / GBK >= 4 && !(force && atoi(force) == 4) && !dst_row && tail_built(epi, t.gamma != nullptr, N);
 }
 
 static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t* wq,
                        const float* sw, const float* bias, void* out, int64_t ldo, int64_t M,
                        int N, int K, hipStream_t stream, const void* residual = nullptr,
                        int64_t ld_res = 0, const int32_t* dst_row = nullptr,
-                       int layout = SAMFAST_LAYOUT_ROWMAJOR) {
+                       int layout = SAMFAST_LAYOUT_ROWMAJOR, const GemmTail* tail = nullptr) {
   // no rows: nothing to do, and the row operands of an empty call may be null
   SF_REQUIRE(wq && (M == 0 || (xq && out)), "gemm_i8: null pointer");
   SF_REQUIRE(layout == SAMFAST_LAYOUT_ROWMAJOR || layout == SAMFAST_LAYOUT_KB64, "gemm_i8: unknown layout %d", layout);
@@ -622,11 +720,42 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   // tiles (proj, lin2: 5) the workgroups that share an X row tile should be adjacent (-23 % / -31 %
   // fetched bytes); with many (qkv 15, lin1 20) 1024 rows per group let W panels be shared
   a.group_m = a.tiles_n <= 6 ? 1 : 1024 / bm;
-  a.stream_out = (epi == EPI_SCALE_BIAS_BF16 || epi == EPI_GELU_BF16) && M * (int64_t)N * 2 >= (256ll << 20);
+  // (an output the quantiser tail reads back right away is not streamed past the caches)
+  a.stream_out = !tail && (epi == EPI_SCALE_BIAS_BF16 || epi == EPI_GELU_BF16) && M * (int64_t)N * 2 >= (256ll << 20);
+  a.tile_counters = nullptr; a.yq = nullptr; a.sy = nullptr; a.ln_gamma = a.ln_beta = nullptr;
+  a.ln_eps = 0.f; a.yq_kb64 = 0;
+  if (tail) {
+    a.tile_counters = tail->counters; a.yq = tail->yq; a.sy = tail->sy;
+    a.ln_gamma = reinterpret_cast<const unsigned short*>(tail->gamma);
+    a.ln_beta = reinterpret_cast<const unsigned short*>(tail->beta);
+    a.ln_eps = tail->eps; a.yq_kb64 = tail->yq_layout == SAMFAST_LAYOUT_KB64;
+  }
   const int64_t total = (int64_t)a.tiles_m * a.tiles_n;
   SF_REQUIRE(total < (1ll << 30), "gemm_i8: too many tiles");
   const unsigned int grid = (unsigned int)(((total + 7) / 8) * 8);
   const bool generic = generic_k;
+  if (tail) {
+    // the caller has checked tail_fusable(): main kernel, 128-row tiles
+#define SF_GEMM_TAIL(E, NN, LN)                                                                              \
+  case NN:                                                                                                   \
+    hipLaunchKernelGGL((gemm_i8_kernel<E, 2, false, NN, LN>), dim3(grid), dim3(256), 0, stream, a);          \
+    break
+    if (epi == EPI_GELU_BF16) {
+      switch (N) {
+        SF_GEMM_TAIL(EPI_GELU_BF16, 3072, false);
+        SF_GEMM_TAIL(EPI_GELU_BF16, 4096, false);
+        SF_GEMM_TAIL(EPI_GELU_BF16, 5120, false);
+      }
+    } else {
+      switch (N) {
+        SF_GEMM_TAIL(EPI_RESIDUAL_BF16, 768, true);
+        SF_GEMM_TAIL(EPI_RESIDUAL_BF16, 1024, true);
+        SF_GEMM_TAIL(EPI_RESIDUAL_BF16, 1280, true);
+      }
+    }
+#undef SF_GEMM_TAIL
+    return check_launch("gemm_i8_kernel (quantiser tail)");
+  }
 #define SF_GEMM_LAUNCH(E)                                                                      \
   do {                                                                                         \
     if (generic)                                                                               \
@@ -686,4 +815,45 @@ extern "C" int samfast_gemm_i8_fused(const int8_t* xq, const float* sx, const in
   }
   return gemm_common(epi, xq, sx, wq, sw, bias, y, ldy, M, N, K,
                      reinterpret_cast<hipStream_t>(stream), residual, ld_res, dst_row, layout);
+}
+
+extern "C" int samfast_gemm_i8_fused_quant(const int8_t* xq, const float* sx, const int8_t* wq,
+                                           const float* sw, const float* bias, void* y, int64_t ldy,
+                                           int64_t M, int N, int K, int dtype, int epilogue,
+                                           const void* residual, int64_t ld_res, int layout,
+                                           const void* ln_gamma, const void* ln_beta, float ln_eps,
+                                           int8_t* yq, float* sy, int yq_layout,
+                                           int32_t* tile_counters, void* stream) {
+  using namespace samfast;
+  if (dtype != SAMFAST_BF16) {
+    set_error("gemm_i8_fused_quant: only bf16 output");
+    return SAMFAST_E_UNSUPPORTED;
+  }
+  int epi;
+  switch (epilogue) {
+    case SAMFAST_EPILOGUE_NONE: epi = EPI_SCALE_BIAS_BF16; break;
+    case SAMFAST_EPILOGUE_GELU: epi = EPI_GELU_BF16; break;
+    case SAMFAST_EPILOGUE_RESIDUAL: epi = EPI_RESIDUAL_BF16; break;
+    default:
+      set_error("gemm_i8_fused_quant: unknown epilogue %d", epilogue);
+      return SAMFAST_E_INVALID;
+  }
+  SF_REQUIRE((ln_gamma == nullptr) == (ln_beta == nullptr), "gemm_i8_fused_quant: gamma and beta go together");
+  SF_REQUIRE(M == 0 || (yq && sy && tile_counters), "gemm_i8_fused_quant: null output or counter pointer");
+  SF_REQUIRE(yq_layout == SAMFAST_LAYOUT_ROWMAJOR || (yq_layout == SAMFAST_LAYOUT_KB64 && N % 64 == 0),
+             "gemm_i8_fused_quant: yq layout must be row-major, or K-block major with N %% 64 == 0");
+  SF_REQUIRE((reinterpret_cast<uintptr_t>(yq) & 7u) == 0 && (reinterpret_cast<uintptr_t>(tile_counters) & 3u) == 0,
+             "gemm_i8_fused_quant: yq must be 8-byte aligned");
+  SF_REQUIRE(!ln_gamma || (aligned16(ln_gamma) && aligned16(ln_beta) && ln_eps > 0.f),
+             "gemm_i8_fused_quant: gamma / beta must be 16-byte aligned and eps positive");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  GemmTail t = {yq, sy, ln_gamma, ln_beta, ln_eps, yq_layout, tile_counters};
+  if (tail_fusable(epi, t, N, K, nullptr))
+    return gemm_common(epi, xq, sx, wq, sw, bias, y, ldy, M, N, K, s, residual, ld_res, nullptr, layout, &t);
+  // shapes the in-kernel quantiser is not built for: the same result from two launches
+  const int rc = gemm_common(epi, xq, sx, wq, sw, bias, y, ldy, M, N, K, s, residual, ld_res, nullptr, layout);
+  if (rc != SAMFAST_OK) return rc;
+  if (ln_gamma)
+    return samfast_layernorm_quant_i8(y, ldy, ln_gamma, ln_beta, ln_eps, nullptr, yq, sy, M, N, dtype, yq_layout, stream);
+  return samfast_quant_rowwise_i8(y, ldy, yq, sy, M, N, dtype, yq_layout, stream);
 }

@@ -15,11 +15,13 @@ Any other input (CPU, fp32, shapes the kernels do not cover) follows the
 reference's own composition through flash_4._attention_rel_h_rel_w.
 
 When, in addition, the four Linears of a Block have been swapped for
-quant.Int8DynamicLinear, Block.forward (:167-183) runs as nine kernel launches with
-no eager glue: LayerNorm + window partition + quantise, qkv GEMM, attention,
-quantise, proj GEMM + window unpartition + residual, LayerNorm + quantise, lin1 GEMM
-+ GELU, quantise, lin2 GEMM + residual.  SAMFAST_FUSED_BLOCK=0 keeps the
-module-by-module composition instead.
+quant.Int8DynamicLinear, Block.forward (:167-183) runs with no eager glue as nine kernel
+launches: LayerNorm + quantise, qkv GEMM, attention, quantise, proj GEMM + residual, LayerNorm
++ quantise, lin1 GEMM + GELU, quantise, lin2 GEMM + residual.  With SAMFAST_FUSED_QUANT=1 the
+three quantisers that follow a GEMM run inside that GEMM (proj + norm2 + quantise, lin1 +
+quantise, lin2 + the NEXT block's norm1 + quantise: five launches per block, same bits; slower
+at the measured shapes, hence not the default).  SAMFAST_FUSED_BLOCK=0 keeps the
+module-by-module composition.
 """
 
 import os
@@ -83,12 +85,27 @@ class ImageEncoderViT(nn.Module):
             LayerNorm2d(out_chans),
         )
 
+    def forward_blocks(self, x: torch.Tensor) -> torch.Tensor:
+        """The transformer blocks on (B, H, W, C) tokens.  Consecutive blocks on the fused int8
+        path are chained: a block's lin2 launch also runs the next block's norm1 and the qkv
+        Linear's quantiser on the rows it has just written."""
+        carry = None
+        for i, blk in enumerate(self.blocks):
+            if not blk._int8_fused_ok(x):
+                x, carry = blk(x), None
+                continue
+            nxt = self.blocks[i + 1] if i + 1 < len(self.blocks) else None
+            next_norm = None
+            if nxt is not None and nxt._int8_fused_ok(x) and nxt._chains_from_previous():
+                next_norm = (nxt.norm1.weight, nxt.norm1.bias, nxt.norm1.eps)
+            x, carry = blk._forward_int8_fused(x, carry, next_norm)
+        return x
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         x = self.patch_embed(x)
         if self.pos_embed is not None:
             x = x + self.pos_embed
-        for blk in self.blocks:
-            x = blk(x)
+        x = self.forward_blocks(x)
         return self.neck(x.permute(0, 3, 1, 2))
 
 
@@ -157,8 +174,17 @@ class Block(nn.Module):
             self._pad_key, self._pad_kv = key, (pk, pv)
         return self._pad_kv
 
-    def _forward_int8_fused(self, x: torch.Tensor) -> torch.Tensor:
-        """image_encoder.py:167-183 with every step on the HIP kernels."""
+    def _chains_from_previous(self) -> bool:
+        """Whether this block's norm1 + quantiser can run in the previous block's lin2 launch:
+        its rows must be the image-ordered tokens (no window gather in front of qkv)."""
+        return self.window_size == 0 or WINDOWS_IN_PLACE
+
+    def _forward_int8_fused(self, x: torch.Tensor, carry=None, next_norm=None):
+        """image_encoder.py:167-183 with every step on the HIP kernels.
+
+        `carry` = (xq, sx): this block's norm1 output, already quantised by the previous block's
+        lin2 launch.  `next_norm` = (gamma, beta, eps) of the next block's norm1: lin2 then
+        also returns that block's carry.  Returns (tokens (B, H, W, C), carry for the next block)."""
         B, H, W, C = x.shape
         attn, mlp = self.attn, self.mlp
         nH = attn.num_heads
@@ -167,6 +193,7 @@ class Block(nn.Module):
         # int8 activations travel K-block major between the quantisers and the GEMMs
         L = _lib.LAYOUT_KB64 if (C % 64 == 0 and KB64_OPERANDS) else _lib.LAYOUT_ROWMAJOR
         ws = self.window_size
+        norm2 = (self.norm2.weight, self.norm2.bias, self.norm2.eps)
         if ws > 0 and not WINDOWS_IN_PLACE:
             # windows materialised: the partition is a row gather in the LayerNorm+quant kernel,
             # the unpartition a row scatter in the proj epilogue
@@ -179,9 +206,14 @@ class Block(nn.Module):
             o = ops.attn_relpos(q, k, v, attn.rel_pos_h, attn.rel_pos_w, (ws, ws), attn.scale)
             oq, so = ops.quant_rowwise(o.permute(0, 2, 1, 3).reshape(Bw * N, C), layout=L)
             tokens = attn.proj.linear_fused(oq, so, _lib.EPILOGUE_RESIDUAL, residual=tokens, dst_row=row_map, layout=L)
+            hq, sh = ops.layernorm_quant(tokens, *norm2, layout=L)
         else:
-            # norm1 + qkv's activation quantiser, qkv GEMM on the image-ordered tokens
-            xq, sx = ops.layernorm_quant(tokens, self.norm1.weight, self.norm1.bias, self.norm1.eps, layout=L)
+            # norm1 + qkv's activation quantiser (unless the previous block's lin2 launch has done
+            # it), qkv GEMM on the image-ordered tokens
+            if carry is not None:
+                xq, sx = carry
+            else:
+                xq, sx = ops.layernorm_quant(tokens, self.norm1.weight, self.norm1.bias, self.norm1.eps, layout=L)
             qkv = attn.qkv.linear_fused(xq, sx, _lib.EPILOGUE_NONE, layout=L).view(B, H * W, 3, nH, hd)
             q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
             if ws > 0:
@@ -194,18 +226,21 @@ class Block(nn.Module):
                 o = ops.attn_relpos(q, k, v, attn.rel_pos_h, attn.rel_pos_w, (H, W), attn.scale)
                 o = o.permute(0, 2, 1, 3).reshape(B * H * W, C)
             oq, so = ops.quant_rowwise(o, layout=L)
-            # proj + `shortcut + x`
-            tokens = attn.proj.linear_fused(oq, so, _lib.EPILOGUE_RESIDUAL, residual=tokens, layout=L)
-        # norm2 + lin1's quantiser, lin1 + GELU, lin2's quantiser, lin2 + `x + mlp(...)`
-        hq, sh = ops.layernorm_quant(tokens, self.norm2.weight, self.norm2.bias, self.norm2.eps, layout=L)
-        h = mlp.lin1.linear_fused(hq, sh, _lib.EPILOGUE_GELU, layout=L)
-        gq, sg = ops.quant_rowwise(h, layout=L)
+            # proj + `shortcut + x`, then norm2 + lin1's quantiser on the rows just written
+            tokens, hq, sh = attn.proj.linear_fused_quant(oq, so, _lib.EPILOGUE_RESIDUAL, residual=tokens,
+                                                          layout=L, ln=norm2, out_layout=L)
+        # lin1 + GELU + lin2's quantiser, lin2 + `x + mlp(...)` (+ the next block's norm1 and quantiser)
+        _, gq, sg = mlp.lin1.linear_fused_quant(hq, sh, _lib.EPILOGUE_GELU, layout=L, out_layout=L)
+        if next_norm is not None:
+            tokens, nq, sn = mlp.lin2.linear_fused_quant(gq, sg, _lib.EPILOGUE_RESIDUAL, residual=tokens,
+                                                         out=tokens, layout=L, ln=next_norm, out_layout=L)
+            return tokens.view(B, H, W, C), (nq, sn)
         tokens = mlp.lin2.linear_fused(gq, sg, _lib.EPILOGUE_RESIDUAL, residual=tokens, out=tokens, layout=L)
-        return tokens.view(B, H, W, C)
+        return tokens.view(B, H, W, C), None
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self._int8_fused_ok(x):
-            return self._forward_int8_fused(x)
+            return self._forward_int8_fused(x)[0]
         shortcut = x
         x = self.norm1(x)
         if self.window_size > 0:

@@ -377,6 +377,84 @@ def gemm_i8_fused(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torc
     return out
 
 
+_tile_counters = {}
+
+
+def tile_counters(rows: int, device) -> torch.Tensor:
+    """The zeroed int32 workspace samfast_gemm_i8_fused_quant wants (one entry per 128 rows), one
+    buffer per (device, stream): every launch leaves it zero again, and launches on one stream
+    cannot overlap."""
+    key = (str(device), torch.cuda.current_stream().cuda_stream)
+    need = -(-rows // 128)
+    buf = _tile_counters.get(key)
+    if buf is None or buf.numel() < need:
+        buf = torch.zeros(max(need, 1024), dtype=torch.int32, device=device)
+        _tile_counters[key] = buf
+    return buf
+
+
+def gemm_i8_fused_quant(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor,
+                        bias: Optional[torch.Tensor], epilogue: int,
+                        residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                        layout: int = _lib.LAYOUT_ROWMAJOR,
+                        ln: Optional[Tuple[torch.Tensor, torch.Tensor, float]] = None,
+                        out_layout: int = _lib.LAYOUT_ROWMAJOR,
+                        counters: Optional[torch.Tensor] = None):
+    """gemm_i8_fused (no row scatter) that also returns its output rows quantised for the next
+    Linear: (y, yq, sy), with yq / sy what quant_rowwise(y) - or, with ln = (gamma, beta, eps),
+    layernorm_quant(y, gamma, beta, eps) - returns, bit for bit, in `out_layout`."""
+    _require_gpu(xq, sx, wq, sw, bias, residual)
+    M, K = _operand_shape(xq, layout)
+    N, Kw = _operand_shape(wq, layout)
+    if K != Kw:
+        raise RuntimeError("samfast: gemm_i8_fused_quant operands disagree on K")
+    if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != M or sw.numel() != N:
+        raise RuntimeError("samfast: scales must be fp32 of length M and N")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N):
+        raise RuntimeError("samfast: bias must be fp32 of length N")
+    if epilogue == _lib.EPILOGUE_RESIDUAL:
+        if residual is None or tuple(residual.shape) != (M, N) or residual.stride(1) != 1 \
+                or residual.dtype != torch.bfloat16:
+            raise RuntimeError("samfast: residual must be a bf16 (M, N) tensor")
+        if out is None:
+            out = torch.empty_like(residual)
+    elif out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=xq.device)
+    if tuple(out.shape) != (M, N) or out.dtype != torch.bfloat16 or out.stride(1) != 1:
+        raise RuntimeError("samfast: out must be a bf16 (M, N) tensor with contiguous rows")
+    gamma = beta = None
+    eps = 0.0
+    if ln is not None:
+        gamma, beta, eps = ln
+        _require_gpu(gamma, beta)
+        if gamma.dtype != torch.bfloat16 or beta.dtype != torch.bfloat16 or gamma.numel() != N or beta.numel() != N:
+            raise RuntimeError("samfast: LayerNorm weight / bias must be bf16 of length N")
+        gamma, beta = gamma.contiguous(), beta.contiguous()
+    yq = _xq_empty(M, N, out_layout, xq.device)
+    sy = torch.empty((M,), dtype=torch.float32, device=xq.device)
+    if counters is None:
+        counters = tile_counters(M, xq.device)
+    if counters.dtype != torch.int32 or counters.numel() * 128 < M or not counters.is_contiguous():
+        raise RuntimeError("samfast: the counter workspace must hold ceil(M / 128) int32")
+    lib = _lib.load()
+    name = {_lib.EPILOGUE_NONE: "gemm_i8_scale_bias", _lib.EPILOGUE_GELU: "gemm_i8_gelu",
+            _lib.EPILOGUE_RESIDUAL: "gemm_i8_residual"}.get(epilogue, "gemm_i8_fused") \
+        + ("_lnquant" if ln is not None else "_quant")
+    code = _timed(
+        name, 2.0 * M * N * K, "op",
+        lambda: lib.samfast_gemm_i8_fused_quant(
+            xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
+            bias.data_ptr() if bias is not None else None, out.data_ptr(), out.stride(0),
+            M, N, K, _lib.SAMFAST_BF16, int(epilogue),
+            residual.data_ptr() if residual is not None else None,
+            residual.stride(0) if residual is not None else 0, int(layout),
+            gamma.data_ptr() if gamma is not None else None,
+            beta.data_ptr() if beta is not None else None, float(eps),
+            yq.data_ptr(), sy.data_ptr(), int(out_layout), counters.data_ptr(), _stream()))
+    _lib.check(code, "gemm_i8_fused_quant")
+    return out, yq, sy
+
+
 def prune24_pack(wq: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """int8 (N, K) -> packed 2:4 form (wc int8 (K/64, N, 32), widx int32 (K/64, N, 2)): per
     aligned group of 4 along K the two largest magnitudes are kept (ties: lowest position).

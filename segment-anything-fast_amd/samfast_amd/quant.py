@@ -17,6 +17,7 @@ inspects shapes keeps working.  Forward needs GPU bf16 activations; there is no
 CPU route.
 """
 
+import os
 from typing import Callable, Optional
 
 import torch
@@ -25,6 +26,14 @@ import torch.nn as nn
 from . import ops
 from ._lib import EPILOGUE_NONE, LAYOUT_KB64, LAYOUT_ROWMAJOR
 from .tools import replace_with_custom_fn_if_matches_filter
+
+# The next Linear's row quantiser inside the producing GEMM (one launch, five per block) or after
+# it (two launches, nine per block).  Both give the same bits.  Measured on the ViT-H batch-16
+# encoder the single launch is the slower one (the workgroup that quantises a row tile holds
+# one of its CU's two GEMM slots for the duration, and the device-scope release of every tile
+# writes the L2 back), so the separate launches are the default; SAMFAST_FUSED_QUANT=1 selects
+# the fused form.
+FUSED_QUANT = os.environ.get("SAMFAST_FUSED_QUANT", "0") != "0"
 
 
 WEIGHT_CONVENTIONS = ("absmax127", "torchao")
@@ -114,6 +123,18 @@ class Int8LinearBase(nn.Module):
                      layout=LAYOUT_ROWMAJOR):
         raise NotImplementedError
 
+    def linear_fused_quant(self, xq, sx, epilogue, residual=None, out=None, layout=LAYOUT_ROWMAJOR,
+                           ln=None, out_layout=LAYOUT_ROWMAJOR):
+        """linear_fused followed by the next Linear's row quantiser (behind a LayerNorm when
+        ln = (gamma, beta, eps) is given): returns (y, yq, sy).  Here as separate launches;
+        Int8DynamicLinear runs all of it inside its GEMM."""
+        y = self.linear_fused(xq, sx, epilogue, residual=residual, out=out, layout=layout)
+        if ln is not None:
+            yq, sy = ops.layernorm_quant(y, ln[0], ln[1], ln[2], layout=out_layout)
+        else:
+            yq, sy = ops.quant_rowwise(y, layout=out_layout)
+        return y, yq, sy
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """The kernels compute on bf16 rows; any other floating input is cast on the way in and
         the result cast back, so the module keeps its input's dtype as nn.Linear does."""
@@ -146,15 +167,27 @@ class Int8DynamicLinear(Int8LinearBase):
                      out: Optional[torch.Tensor] = None, layout: int = LAYOUT_ROWMAJOR) -> torch.Tensor:
         """The GEMM + epilogue on already quantised rows (see ops.gemm_i8_fused); `layout` is
         the layout xq comes in.  The K-block major copy of the weight is made on first use."""
-        if layout == LAYOUT_KB64:
-            key = (self.wq.data_ptr(), self.wq._version, str(self.wq.device))
-            if self._wq_kb64 is None or self._wq_kb64_key != key:  # rebuilt after load_state_dict / .to()
-                self._wq_kb64, self._wq_kb64_key = ops.to_kb64(self.wq), key
-            w = self._wq_kb64
-        else:
-            w = self.wq
-        return ops.gemm_i8_fused(xq, sx, w, self.sw, self.bias_f32, epilogue,
+        return ops.gemm_i8_fused(xq, sx, self._weight_for(layout), self.sw, self.bias_f32, epilogue,
                                  residual=residual, dst_row=dst_row, out=out, layout=layout)
+
+    def _weight_for(self, layout: int) -> torch.Tensor:
+        if layout != LAYOUT_KB64:
+            return self.wq
+        key = (self.wq.data_ptr(), self.wq._version, str(self.wq.device))
+        if self._wq_kb64 is None or self._wq_kb64_key != key:  # rebuilt after load_state_dict / .to()
+            self._wq_kb64, self._wq_kb64_key = ops.to_kb64(self.wq), key
+        return self._wq_kb64
+
+    def linear_fused_quant(self, xq, sx, epilogue, residual=None, out=None, layout=LAYOUT_ROWMAJOR,
+                           ln=None, out_layout=LAYOUT_ROWMAJOR):
+        """GEMM + epilogue + the next Linear's quantiser as one launch (ops.gemm_i8_fused_quant);
+        FUSED_QUANT = False keeps the quantiser a launch of its own (same results)."""
+        if not FUSED_QUANT:
+            return super().linear_fused_quant(xq, sx, epilogue, residual=residual, out=out, layout=layout,
+                                              ln=ln, out_layout=out_layout)
+        return ops.gemm_i8_fused_quant(xq, sx, self._weight_for(layout), self.sw, self.bias_f32, epilogue,
+                                       residual=residual, out=out, layout=layout, ln=ln,
+                                       out_layout=out_layout)
 
     def extra_repr(self) -> str:
         return f"in_features={self.in_features}, out_features={self.out_features}, int8 dynamic"

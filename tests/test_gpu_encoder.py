@@ -232,9 +232,7 @@ def _trunk_input(enc, images):
 
 
 def _run_blocks(enc, x):
-    for blk in enc.blocks:
-        x = blk(x)
-    return x
+    return enc.forward_blocks(x)
 
 
 def test_vit_h_all_32_blocks_vs_oracle():
@@ -312,3 +310,31 @@ def test_vit_h_batch_32_sparse_mlp_bitwise_equals_dense_kernels_on_pruned_weight
     torch.cuda.synchronize()
     assert torch.isfinite(ya.float()).all()
     assert torch.equal(ya.view(torch.int16), yb.view(torch.int16))
+
+
+def test_chained_blocks_equal_separate_quantiser_launches(monkeypatch):
+    """The encoder's blocks with every row quantiser inside the GEMM that produces its rows (five
+    launches per block, blocks chained through lin2) against the same blocks with the quantisers as
+    launches of their own, and against blocks called one by one: bit-equal."""
+    from samfast_amd import apply_dynamic_quant, quant
+    from samfast_amd.modeling import ImageEncoderViT
+    from samfast_amd.synthetic import init_encoder_weights, make_images
+    enc = ImageEncoderViT(depth=4, embed_dim=1280, num_heads=16, global_attn_indexes=(1, 3),
+                          window_size=14, use_rel_pos=True, mlp_ratio=4,
+                          norm_layer=partial(torch.nn.LayerNorm, eps=1e-6))
+    init_encoder_weights(enc, seed=6)
+    enc = enc.eval().to(torch.bfloat16).cuda()
+    apply_dynamic_quant(enc)
+    with torch.no_grad():
+        x0 = _trunk_input(enc, make_images(3, seed=2).to(torch.bfloat16).cuda())
+        monkeypatch.setattr(quant, "FUSED_QUANT", True)
+        chained = enc.forward_blocks(x0.clone())
+        one_by_one = x0.clone()
+        for blk in enc.blocks:
+            one_by_one = blk(one_by_one)
+        monkeypatch.setattr(quant, "FUSED_QUANT", False)
+        separate = enc.forward_blocks(x0.clone())
+    torch.cuda.synchronize()
+    assert torch.isfinite(chained.float()).all()
+    assert torch.equal(chained.view(torch.int16), separate.view(torch.int16))
+    assert torch.equal(chained.view(torch.int16), one_by_one.view(torch.int16))

@@ -409,3 +409,71 @@ def test_layernorm_quant_statistics_against_float64(K, mean, std):
     err = (q * s[:, None] - y64).abs()
     bound = 0.5 * s[:, None] + y64.abs() * (2.0 ** -8 + 1e-4) + 1e-4
     assert (err <= bound).all(), (err - bound).max().item()
+
+
+def _fused_quant_case(M, N, K, epilogue, ln, seed, layout):
+    """Inputs of one gemm_i8_fused_quant call and the results of the separate launches it must equal."""
+    from samfast_amd import _lib, ops
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((M, K), generator=g)
+    x[torch.randperm(M, generator=g)[:max(1, M // 1000)]] *= 20.0
+    w = torch.randn((N, K), generator=g) * 0.02
+    bias = (torch.randn((N,), generator=g) * 0.02).cuda()
+    xq, sx = ops.quant_rowwise(x.to(torch.bfloat16).cuda(), layout)
+    wq, sw = ops.quant_rowwise(w.to(torch.bfloat16).cuda(), layout)
+    res = torch.randn((M, N), generator=g).to(torch.bfloat16).cuda() if epilogue == _lib.EPILOGUE_RESIDUAL else None
+    norm = None
+    if ln:
+        norm = ((1 + 0.1 * torch.randn(N, generator=g)).to(torch.bfloat16).cuda(),
+                (0.1 * torch.randn(N, generator=g)).to(torch.bfloat16).cuda(), 1e-6)
+    y_ref = ops.gemm_i8_fused(xq, sx, wq, sw, bias, epilogue, residual=res, layout=layout)
+    if ln:
+        q_ref, s_ref = ops.layernorm_quant(y_ref, norm[0], norm[1], norm[2], layout=layout)
+    else:
+        q_ref, s_ref = ops.quant_rowwise(y_ref, layout=layout)
+    return (xq, sx, wq, sw, bias, res, norm), (y_ref, q_ref, s_ref)
+
+
+@pytest.mark.parametrize("M,N,K,kind", [
+    (65536, 5120, 1280, "gelu"), (65536, 1280, 1280, "ln"), (65536, 1280, 5120, "ln"),   # the ViT-H linears
+    (4096, 3072, 768, "gelu"), (4096, 768, 3072, "ln"), (8192, 1024, 1024, "ln"),        # ViT-B / ViT-L widths
+    (1, 1280, 1280, "ln"), (127, 5120, 1280, "gelu"), (129, 1280, 1280, "ln"), (1000, 5120, 1280, "gelu"),
+    (300, 1280, 128, "ln"),      # fewer k tiles than LDS stages: runs as two launches
+    (300, 2048, 1280, "gelu"),   # a width the in-kernel quantiser is not built for: two launches
+    (300, 1280, 1280, "plain_after_residual"),
+])
+def test_gemm_with_output_quantiser_equals_separate_launches(M, N, K, kind):
+    """The GEMM that also quantises its output rows for the next Linear (inside the kernel: the
+    workgroup that completes a row tile does it) against the separate launches: y, codes and scales
+    bit-equal, in both operand layouts; the counter workspace is all zero again afterwards and a
+    second call on the same workspace gives the same result."""
+    from samfast_amd import _lib, ops
+    print(f"case fused quant M={M} N={N} K={K} {kind}", flush=True)
+    epilogue = _lib.EPILOGUE_GELU if kind == "gelu" else _lib.EPILOGUE_RESIDUAL
+    ln = kind == "ln"
+    for layout in (_lib.LAYOUT_KB64, _lib.LAYOUT_ROWMAJOR) if M <= 8192 else (_lib.LAYOUT_KB64,):
+        (xq, sx, wq, sw, bias, res, norm), (y_ref, q_ref, s_ref) = _fused_quant_case(M, N, K, epilogue, ln, M + N + K, layout)
+        counters = torch.zeros(-(-M // 128), dtype=torch.int32, device="cuda")
+        for rep in range(2):
+            y, q, s = ops.gemm_i8_fused_quant(xq, sx, wq, sw, bias, epilogue, residual=res, layout=layout,
+                                              ln=norm, out_layout=layout, counters=counters)
+            torch.cuda.synchronize()
+            assert torch.equal(y.view(torch.int16), y_ref.view(torch.int16)), (layout, rep)
+            assert torch.equal(s.view(torch.int32), s_ref.view(torch.int32)), (layout, rep)
+            assert torch.equal(q, q_ref), (layout, rep)
+            assert int(counters.abs().sum()) == 0
+        del y, q, s, y_ref, q_ref, s_ref, xq, wq, res
+
+
+def test_gemm_with_output_quantiser_in_place_residual():
+    """lin2's form: the output overwrites the residual stream it reads (out = residual)."""
+    from samfast_amd import _lib, ops
+    L = _lib.LAYOUT_KB64
+    (xq, sx, wq, sw, bias, res, norm), (y_ref, q_ref, s_ref) = _fused_quant_case(
+        2048, 1280, 5120, _lib.EPILOGUE_RESIDUAL, True, 11, L)
+    buf = res.clone()
+    y, q, s = ops.gemm_i8_fused_quant(xq, sx, wq, sw, bias, _lib.EPILOGUE_RESIDUAL, residual=buf, out=buf,
+                                      layout=L, ln=norm, out_layout=L)
+    assert y.data_ptr() == buf.data_ptr()
+    assert torch.equal(y.view(torch.int16), y_ref.view(torch.int16))
+    assert torch.equal(q, q_ref) and torch.equal(s.view(torch.int32), s_ref.view(torch.int32))
