@@ -231,6 +231,23 @@ int samfast_gemm_i8_fused_quant(
     int8_t* yq, float* sy, int yq_layout, int32_t* tile_counters, void* stream);
 
 /*
+ * samfast_gemm_i8_fused_quant for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops, harnesses that forbid it).  It has no counterpart in the reference.  Same
+ * arguments and results, minus the `tile_counters` workspace: the counters live in a device array
+ * inside the library (128 KiB per GPU, held until the process ends), whose entries the call clears
+ * with a small kernel before it uses them.  M is limited to 4 194 304 rows (32768 row tiles of 128);
+ * a larger M returns SAMFAST_E_INVALID.  All calls on one GPU share that array, so two such calls
+ * must not overlap in time on one GPU (issue them on one stream, or order the streams).
+ */
+int samfast_gemm_i8_fused_quant_noalloc(
+    const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
+    const float* bias, void* y, int64_t ldy,
+    int64_t M, int N, int K, int dtype, int epilogue,
+    const void* residual, int64_t ld_res, int layout,
+    const void* ln_gamma, const void* ln_beta, float ln_eps,
+    int8_t* yq, float* sy, int yq_layout, void* stream);
+
+/*
  * 2:4-sparse weights for the sparse int8 matrix cores (v_smfmac_i32_32x32x64_i8).
  *
  * samfast_prune24_pack_i8: from a dense int8 weight wq (N, K) keep, in every aligned group

@@ -50,6 +50,7 @@
 // counter back to zero for the next launch.  The other workgroup resident on the CU keeps the
 // matrix pipe busy meanwhile.
 #include "quant_row.hpp"
+#include <pthread.h>
 #include <stdlib.h>
 #include <type_traits>
 
@@ -856,4 +857,72 @@ extern "C" int samfast_gemm_i8_fused_quant(const int8_t* xq, const float* sx, co
   if (ln_gamma)
     return samfast_layernorm_quant_i8(y, ldy, ln_gamma, ln_beta, ln_eps, nullptr, yq, sy, M, N, dtype, yq_layout, stream);
   return samfast_quant_rowwise_i8(y, ldy, yq, sy, M, N, dtype, yq_layout, stream);
+}
+
+// ---- the same call for callers that cannot allocate ---------------------------------------
+// The counter workspace of samfast_gemm_i8_fused_quant lives in a file-scope device array, one
+// copy per GPU, held until the process ends.  Its address on a device is looked up once per
+// device (the array's name is only a host-side handle, never a device address).
+namespace samfast {
+
+constexpr int kNoAllocMaxTiles = 32768;  // 128 KiB per GPU: up to 32768 * 128 = 4 194 304 rows
+constexpr int kNoAllocMaxDevices = 64;
+static __device__ __align__(256) int32_t scratch[kNoAllocMaxTiles];
+
+static int32_t* g_scratch_ptr[kNoAllocMaxDevices];  // per device, null until looked up
+static pthread_mutex_t g_scratch_lock = PTHREAD_MUTEX_INITIALIZER;
+
+// address of `scratch` on the current device, looked up on the first call per device
+static int scratch_of_current_device(int32_t** out) {
+  int dev = -1;
+  const hipError_t e0 = hipGetDevice(&dev);
+  if (e0 != hipSuccess) SF_FAIL(SAMFAST_E_LAUNCH, "gemm_i8_fused_quant_noalloc: hipGetDevice: %s", hipGetErrorString(e0));
+  SF_REQUIRE(dev >= 0 && dev < kNoAllocMaxDevices, "gemm_i8_fused_quant_noalloc: device index %d out of range", dev);
+  pthread_mutex_lock(&g_scratch_lock);
+  int32_t* p = g_scratch_ptr[dev];
+  hipError_t e1 = hipSuccess;
+  if (!p) {
+    e1 = hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch));
+    if (e1 == hipSuccess) g_scratch_ptr[dev] = p;
+  }
+  pthread_mutex_unlock(&g_scratch_lock);
+  if (e1 != hipSuccess || !p)
+    SF_FAIL(SAMFAST_E_LAUNCH, "gemm_i8_fused_quant_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e1));
+  *out = p;
+  return SAMFAST_OK;
+}
+
+// the counters a launch is about to use start at zero whatever an earlier call left behind
+// (a fill kernel rather than a memset node: the call may be recorded into a graph)
+__global__ void clear_counters_kernel(int32_t* counters, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0;
+}
+
+}  // namespace samfast
+
+extern "C" int samfast_gemm_i8_fused_quant_noalloc(const int8_t* xq, const float* sx, const int8_t* wq,
+                                                   const float* sw, const float* bias, void* y, int64_t ldy,
+                                                   int64_t M, int N, int K, int dtype, int epilogue,
+                                                   const void* residual, int64_t ld_res, int layout,
+                                                   const void* ln_gamma, const void* ln_beta, float ln_eps,
+                                                   int8_t* yq, float* sy, int yq_layout, void* stream) {
+  using namespace samfast;
+  SF_REQUIRE(M >= 0, "gemm_i8_fused_quant_noalloc: bad M=%lld", (long long)M);
+  const int64_t tiles = (M + 127) / 128;
+  SF_REQUIRE(tiles <= kNoAllocMaxTiles,
+             "gemm_i8_fused_quant_noalloc: M=%lld needs %lld row-tile counters, the built-in workspace holds %d "
+             "(at most %lld rows); use samfast_gemm_i8_fused_quant with a workspace of your own",
+             (long long)M, (long long)tiles, kNoAllocMaxTiles, (long long)kNoAllocMaxTiles * 128);
+  int32_t* counters = nullptr;
+  const int rc = scratch_of_current_device(&counters);
+  if (rc != SAMFAST_OK) return rc;
+  if (tiles > 0) {
+    hipLaunchKernelGGL(clear_counters_kernel, dim3((unsigned int)((tiles + 255) / 256)), dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(stream), counters, (int)tiles);
+    const int rl = check_launch("clear_counters_kernel");
+    if (rl != SAMFAST_OK) return rl;
+  }
+  return samfast_gemm_i8_fused_quant(xq, sx, wq, sw, bias, y, ldy, M, N, K, dtype, epilogue, residual, ld_res,
+                                     layout, ln_gamma, ln_beta, ln_eps, yq, sy, yq_layout, counters, stream);
 }

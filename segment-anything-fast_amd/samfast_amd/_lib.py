@@ -38,6 +38,9 @@ _SIGNATURES = {
     "samfast_gemm_i8_fused_quant": (
         _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _i32,
                _ptr, _i64, _i32, _ptr, _ptr, _f32, _ptr, _ptr, _i32, _ptr, _ptr]),
+    "samfast_gemm_i8_fused_quant_noalloc": (
+        _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _i32,
+               _ptr, _i64, _i32, _ptr, _ptr, _f32, _ptr, _ptr, _i32, _ptr]),
     "samfast_prune24_pack_i8": (_i32, [_ptr, _ptr, _ptr, _i32, _i32, _ptr]),
     "samfast_gemm_i8_sparse24_i32": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _i32, _i32, _ptr]),
     "samfast_gemm_i8_sparse24_fused": (
