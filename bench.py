@@ -188,6 +188,7 @@ def mfma_ceiling():
     operands = {
         0: {"zeros": torch.zeros(n8, dtype=torch.int8, device=dev),
             "small_ints": torch.randint(0, 3, (n8,), generator=g, dtype=torch.int8, device=dev),
+            "gaussian_codes": (torch.randn(n8, generator=g, device=dev) * 28).round().clamp(-127, 127).to(torch.int8),
             "random_int8": torch.randint(-127, 128, (n8,), generator=g, dtype=torch.int8, device=dev)},
         1: {"zeros": torch.zeros(n8 // 2, dtype=torch.bfloat16, device=dev),
             "ones": torch.ones(n8 // 2, dtype=torch.bfloat16, device=dev),
@@ -214,6 +215,34 @@ def mfma_ceiling():
                 torch.cuda.synchronize()
                 best = max(best, ops.value / (e0.elapsed_time(e1) * 1e-3) / 1e15)
             res[key][name] = round(best, 3)
+    # the same question asked of the real GEMM kernel: one encoder shape (qkv, 65536 x 3840 x 1280,
+    # scale + bias epilogue) on all-zero codes and on codes like the encoder's, ten launches back to back
+    from samfast_amd import ops
+    M, N, K = 65536, 3840, 1280
+    sx = torch.full((M,), 0.01, device=dev)
+    sw = torch.full((N,), 0.001, device=dev)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    gemm = {"what": f"gemm_i8 {M}x{N}x{K}, scale + bias -> bf16, 10 launches back to back", "unit": "POP/s"}
+    for name in ("zeros", "gaussian_codes"):
+        if name == "zeros":
+            xq = torch.zeros((K // 64, M, 64), dtype=torch.int8, device=dev)
+            wq = torch.zeros((K // 64, N, 64), dtype=torch.int8, device=dev)
+        else:
+            xq = (torch.randn((K // 64, M, 64), device=dev, generator=g) * 28).round().clamp(-127, 127).to(torch.int8)
+            wq = (torch.randn((K // 64, N, 64), device=dev, generator=g) * 28).round().clamp(-127, 127).to(torch.int8)
+        run = lambda: ops.gemm_i8_fused(xq, sx, wq, sw, None, _lib.EPILOGUE_NONE, out=y, layout=_lib.LAYOUT_KB64)
+        for _ in range(3):
+            run()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        gemm[name] = round(2.0 * M * N * K * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e15, 3)
+        del xq, wq
+    res["gemm_i8_kernel_same_shape_different_data"] = gemm
     return res
 
 

@@ -477,3 +477,35 @@ def test_gemm_with_output_quantiser_in_place_residual():
     assert y.data_ptr() == buf.data_ptr()
     assert torch.equal(y.view(torch.int16), y_ref.view(torch.int16))
     assert torch.equal(q, q_ref) and torch.equal(s.view(torch.int32), s_ref.view(torch.int32))
+
+
+@pytest.mark.parametrize("M,N,K,epi", [(300, 1280, 1280, "residual"), (1000, 3840, 1280, "none"),
+                                       (513, 5120, 1280, "gelu"), (260, 1280, 5120, "residual_scatter")])
+def test_gemm_two_and_three_workgroups_per_cu_agree(monkeypatch, M, N, K, epi):
+    """The main GEMM kernel exists in two forms - three workgroups per CU (single-buffered fragments,
+    two LDS stages, epilogue staged in two halves; the default) and two per CU (SAMFAST_GEMM_WG3=0) -
+    that must agree bit for bit with each other (and, by the other tests, with the oracle)."""
+    from samfast_amd import _lib, ops
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).cuda()
+    bias = (torch.randn((N,), generator=g) * 0.02).cuda()
+    L = _lib.LAYOUT_KB64
+    xq, sx = ops.quant_rowwise(x, L)
+    wq, sw = ops.quant_rowwise(w, L)
+    kw = {}
+    code = {"none": _lib.EPILOGUE_NONE, "gelu": _lib.EPILOGUE_GELU}.get(epi, _lib.EPILOGUE_RESIDUAL)
+    if code == _lib.EPILOGUE_RESIDUAL:
+        rows = M + 40 if epi == "residual_scatter" else M
+        kw["residual"] = torch.randn((rows, N), generator=g).to(torch.bfloat16).cuda()
+        if epi == "residual_scatter":
+            perm = torch.randperm(rows, generator=g)[:M].to(torch.int32)
+            perm[5] = -1
+            kw["dst_row"] = perm.cuda()
+    outs = []
+    for wg3 in ("1", "0"):
+        monkeypatch.setenv("SAMFAST_GEMM_WG3", wg3)
+        out = torch.zeros_like(kw["residual"]) if "residual" in kw else None
+        outs.append(ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L, out=out, **kw).clone())
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
