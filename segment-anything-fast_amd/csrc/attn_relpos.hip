@@ -722,12 +722,12 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     const u32x4 one = {0x3F80u, 0u, 0u, 0u};
     *reinterpret_cast<u32x4*>(vl + (tid * C::VSTR + HD) * 2) = one;
   }
-  if (!has_tile) {  // the eighth wavefront only helps with the staging
+  if (!has_tile) {  // a wavefront without a query tile only helps with the staging and with the output
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    return;
+    __syncthreads();  // V complete (the barrier the others reach after their first score tile)
   }
 
+  if (has_tile) {
   // V^T operand through transposing LDS reads (ds_read_b64_tr_b16): in each group of 16 lanes,
   // lane l receives as element j the l%4-th 16-bit value of the 8 bytes addressed by lane
   // 4j + l/4.  Source lane 4j + i points at key j of the lane half's four keys, channels
@@ -838,9 +838,14 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     l = l_run + xor32(l_run);
   }
   const float inv = 1.0f / l;
-  const int otok = qi < N ? tok_of(qi) : -1;  // padding queries produce no output
-  if (otok >= 0) {
-    unsigned short* op = a.out + b * a.o_sb + h * a.o_sh + (int64_t)otok * a.o_sn;
+  // ---- output: through LDS, so that a token's HD channels leave as one contiguous run ----------
+  // Written straight from the accumulators a lane would store 8 bytes to each of 32 different
+  // token rows per instruction; staged as (token, channel) rows in the K area - free once every
+  // wavefront has left its key loop - the whole workgroup then writes 16 bytes per lane with the
+  // HD/8 pieces of a token in neighbouring lanes.
+  __syncthreads();
+  if (qi < N) {
+    unsigned char* orow_l = kl + qi * (C::KSTR * 2);
 #pragma unroll
     for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
@@ -849,9 +854,27 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
         if (d < HD) {
           const u32x2 o = {pack_bf16x2(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
                            pack_bf16x2(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
-          *reinterpret_cast<u32x2*>(op + d) = o;
+          *reinterpret_cast<u32x2*>(orow_l + d * 2) = o;
         }
       }
+  }
+  }  // has_tile
+  else {
+    __syncthreads();  // the key loops are over: the K area becomes the output staging area
+  }
+  __syncthreads();    // the staged output is complete
+  {
+    constexpr int PPT = HD / 8;  // 16-byte pieces per token
+    unsigned short* obase = a.out + b * a.o_sb + h * a.o_sh;
+    for (int p = tid; p < N * PPT; p += C::THREADS) {
+      const int n = (p * (65536 / PPT + 1)) >> 16;  // p / PPT, exact for p < 4096
+      const int col = p - n * PPT;
+      const int otok = tok_of(n);  // padding tokens produce no output
+      if (otok >= 0) {
+        const u32x4 o = *reinterpret_cast<const u32x4*>(kl + n * (C::KSTR * 2) + col * 16);
+        *reinterpret_cast<u32x4*>(obase + (int64_t)otok * a.o_sn + col * 8) = o;
+      }
+    }
   }
 }
 
