@@ -42,7 +42,7 @@ PEAK = {"op": ("mfma", 5.0e15, "TOP/s"),       # int8 dense MFMA
 # workload (vit_h, batch 16, dense int8 linears) and only while the kernel's source file still
 # has the hash it had when the counters were taken (otherwise `traffic` is null).
 TRAFFIC_SOURCE = "profiles/bench_vit_h_bs16_pmc_traffic.txt"
-TRAFFIC = {"gemm_i8_kernel": (1.0587e9, "gemm_i8.hip", "e6c828909dfa3b6e")}
+TRAFFIC = {"gemm_i8_kernel": (1.0259e9, "gemm_i8.hip", "16e4fb6bc761b8b3")}
 
 
 def parse():
@@ -194,6 +194,10 @@ def mfma_ceiling():
             "ones": torch.ones(n8 // 2, dtype=torch.bfloat16, device=dev),
             "random_normal": torch.randn(n8 // 2, generator=g, device=dev).to(torch.bfloat16)},
     }
+    # the same codes without their signs, and one (A, B) pair repeated for every instruction
+    operands[0]["gaussian_codes_non_negative"] = operands[0]["gaussian_codes"].abs()
+    operands[0]["random_int8_same_pair_every_instruction"] = \
+        operands[0]["random_int8"].view(4, -1)[:1].repeat(4, 1).reshape(-1).contiguous()
     res = {"what": "8 independent MFMAs per round and wavefront, operands in registers, 512 workgroups of "
                    "4 wavefronts (2 wavefronts per SIMD on 256 CUs), ~40 ms per launch, events on the launch stream",
            "int8_v_mfma_i32_32x32x32_i8": {"unit": "POP/s", "published_peak": 5.0},
