@@ -33,9 +33,11 @@ extern "C" {
 
 #define SAMFAST_VERSION 1
 
-/* element type of attention operands / linear outputs: bf16 is the only one built (other
- * values of a `dtype` argument return SAMFAST_E_UNSUPPORTED) */
+/* element types (`dtype` arguments).  The attention entry points take both, as the reference's
+ * operator does (flash_4.py:188,348); the int8 linears read and write bf16 only and return
+ * SAMFAST_E_UNSUPPORTED for anything else. */
 #define SAMFAST_BF16 0
+#define SAMFAST_F16 1
 
 #define SAMFAST_OK 0
 #define SAMFAST_E_INVALID (-1)      /* bad shape / stride / alignment / null pointer */
@@ -75,7 +77,8 @@ const char* samfast_last_error(void);
  * rel_pos_h: (2*gh-1, hd) contiguous, rel_pos_w: (2*gw-1, hd) contiguous, same
  *   element type as q.
  * Supported: hd in {64, 80}; (gw == 64 and N % 128 == 0) or (gh <= 15 and
- *   gw <= 16 and N <= 208); dtype SAMFAST_BF16.
+ *   gw <= 16 and N <= 208); dtype SAMFAST_BF16 or SAMFAST_F16 (q, k, v, out and the tables
+ *   all of that type; accumulation, softmax and bias in fp32 either way).
  */
 int samfast_attn_relpos_fwd(
     const void* q, const void* k, const void* v,
@@ -96,7 +99,7 @@ int samfast_attn_relpos_fwd(
  * the reference's zero-padded tokens: they take part as keys / values with the rows
  * pad_k / pad_v ((nH, hd) each, same element type - for SAM the bf16-rounded k and v bias of
  * the qkv Linear, which is what a zero input row produces) and produce no output.
- * rel_pos_h / rel_pos_w: (2*ws-1, hd).  Supported: hd in {64, 80}, ws <= 14 (ws*ws <= 208), bf16.
+ * rel_pos_h / rel_pos_w: (2*ws-1, hd).  Supported: hd in {64, 80}, ws <= 14 (ws*ws <= 208), bf16 or fp16.
  */
 int samfast_attn_relpos_windowed_fwd(
     const void* q, const void* k, const void* v,

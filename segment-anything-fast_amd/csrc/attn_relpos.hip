@@ -69,17 +69,45 @@ struct AttnArgs {
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLazyLog2 = 8.0f;  // softmax reference lags the running maximum by at most 2^8
 
-SF_DEVICE bf16x8 as_bf16x8(u32x4 w) { return __builtin_bit_cast(bf16x8, w); }
+// The two 16-bit element types of q / k / v / out (and of the bias factors): what differs between
+// them is the matrix instruction, the conversions and three bit patterns.  Eight elements travel
+// as four 32-bit words (u32x4) everywhere outside these functions.
+struct ElemBf16 {
+  static constexpr unsigned int kOne = 0x3F80u;   // 1.0
+  static constexpr unsigned int kMask = 0xF149u;  // -1e30: added to a score (before the scale), it removes the key
+  static SF_DEVICE f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static SF_DEVICE unsigned int pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+  static SF_DEVICE float lo(unsigned int w) { return bf16_lo_to_f32(w); }
+  static SF_DEVICE float hi(unsigned int w) { return bf16_hi_to_f32(w); }
+  static SF_DEVICE float from_bits(unsigned short h) { return bf16_bits_to_f32(h); }
+};
+struct ElemF16 {
+  typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  static constexpr unsigned int kOne = 0x3C00u;   // 1.0
+  static constexpr unsigned int kMask = 0xFB53u;  // -60000 (fp16 ends at 65504): times scale*log2(e) still below -2^12
+  static SF_DEVICE f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static SF_DEVICE unsigned int pack2(float lo, float hi) {  // round to nearest even
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, f16x2));
+  }
+  static SF_DEVICE float from_bits(unsigned short h) { return (float)__builtin_bit_cast(_Float16, h); }
+  static SF_DEVICE float lo(unsigned int w) { return from_bits((unsigned short)(w & 0xffffu)); }
+  static SF_DEVICE float hi(unsigned int w) { return from_bits((unsigned short)(w >> 16)); }
+};
 
-SF_DEVICE bf16x8 load_bf16x8_global(const unsigned short* p) {
-  return as_bf16x8(*reinterpret_cast<const u32x4*>(p));
-}
+SF_DEVICE u32x4 load_x8_global(const unsigned short* p) { return *reinterpret_cast<const u32x4*>(p); }
 
-SF_DEVICE bf16x8 cvt_bf16x8(const f32x16& s, int base) {
+template <typename T>
+SF_DEVICE u32x4 cvt_x8(const f32x16& s, int base) {
   u32x4 w;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(s[base + 2 * i], s[base + 2 * i + 1]);
-  return as_bf16x8(w);
+  for (int i = 0; i < 4; ++i) w[i] = T::pack2(s[base + 2 * i], s[base + 2 * i + 1]);
+  return w;
 }
 
 // max(v, v of lane ^ 32) without an LDS round trip: v_permlane32_swap exchanges the upper half
@@ -130,7 +158,7 @@ struct GlobalCfg {
   static_assert(X_BYTES <= LDS_BYTES, "gather scratch must fit in the workgroup's LDS");
 };
 
-template <int HD, int QT, bool FUSED, int WAVES>
+template <typename T, int HD, int QT, bool FUSED, int WAVES>
 __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_kernel(AttnArgs a) {
   using C = GlobalCfg<HD, QT, WAVES>;
   __shared__ __attribute__((aligned(16))) unsigned char lds[C::LDS_BYTES];
@@ -226,12 +254,12 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
   };
 
   // ---- Q^T operand: lane holds query lr of tile t, channels 16s + 8lh .. +7 ----
-  bf16x8 qf[QT][C::KS];
+  u32x4 qf[QT][C::KS];
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
     const unsigned short* qp = qbase + (int64_t)(q_wg + q_wave + 32 * t + lr) * a.q_sn + 8 * lh;
 #pragma unroll
-    for (int s = 0; s < C::KS; ++s) qf[t][s] = load_bf16x8_global(qp + 16 * s);
+    for (int s = 0; s < C::KS; ++s) qf[t][s] = load_x8_global(qp + 16 * s);
   }
 
   // ---- bias prologue -----------------------------------------------------------
@@ -241,7 +269,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
   auto first_tile = [&]() {
     if (C::ONES_ROW && tid < 128) {  // spare piece of every V row of both stages: (1, 0, .., 0)
       const int buf = tid >> 6, row = tid & 63;
-      const u32x4 one = {0x3F80u, 0u, 0u, 0u};
+      const u32x4 one = {T::kOne, 0u, 0u, 0u};
       *reinterpret_cast<u32x4*>(lds + buf * C::STAGE + C::KBYTES + (row * C::VSTR + HD) * 2) = one;
     }
     stage_dma(0, 0);
@@ -261,8 +289,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
         for (int s = 0; s < C::KS; ++s) {
-          const bf16x8 av = load_bf16x8_global(th + trow * HD + 16 * s + 8 * lh);
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[t][s], acc, 0, 0, 0);
+          const u32x4 av = load_x8_global(th + trow * HD + 16 * s + 8 * lh);
+          acc = T::mfma(av, qf[t][s], acc);
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -290,8 +318,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
           for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
           for (int s = 0; s < C::KS; ++s) {
-            const bf16x8 av = load_bf16x8_global(tw + trow * HD + 16 * s + 8 * lh);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[t][s], acc, 0, 0, 0);
+            const u32x4 av = load_x8_global(tw + trow * HD + 16 * s + 8 * lh);
+            acc = T::mfma(av, qf[t][s], acc);
           }
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
@@ -321,7 +349,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
     const unsigned short* rhb = a.rh + b * a.rh_sb + h * a.rh_sh + (int64_t)q_wg * a.rh_sn;
     for (int idx = tid; idx < C::BM * a.gh; idx += 64 * WAVES) {
       const int ql = idx % C::BM, kh = idx / C::BM;
-      relhT[kh * C::BM + ql] = bf16_bits_to_f32(rhb[(int64_t)ql * a.rh_sn + kh]) * kLog2e;
+      relhT[kh * C::BM + ql] = T::from_bits(rhb[(int64_t)ql * a.rh_sn + kh]) * kLog2e;
     }
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
@@ -332,10 +360,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const u32x2 w = *reinterpret_cast<const u32x2*>(rwp + 32 * nt + 8 * j + 4 * lh);
-          b1[t][nt][4 * j + 0] = bf16_lo_to_f32(w[0]) * a.inv_scale;
-          b1[t][nt][4 * j + 1] = bf16_hi_to_f32(w[0]) * a.inv_scale;
-          b1[t][nt][4 * j + 2] = bf16_lo_to_f32(w[1]) * a.inv_scale;
-          b1[t][nt][4 * j + 3] = bf16_hi_to_f32(w[1]) * a.inv_scale;
+          b1[t][nt][4 * j + 0] = T::lo(w[0]) * a.inv_scale;
+          b1[t][nt][4 * j + 1] = T::hi(w[0]) * a.inv_scale;
+          b1[t][nt][4 * j + 2] = T::lo(w[1]) * a.inv_scale;
+          b1[t][nt][4 * j + 3] = T::hi(w[1]) * a.inv_scale;
         }
     }
   }
@@ -368,11 +396,11 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
       // the two key half-tiles are independent accumulator chains: alternate them
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
-        const bf16x8 av = as_bf16x8(*reinterpret_cast<const u32x4*>(
-            kl + ((32 * nt + lr) * C::KSTR + 16 * ks + 8 * lh) * 2));
+        const u32x4 av = *reinterpret_cast<const u32x4*>(
+            kl + ((32 * nt + lr) * C::KSTR + 16 * ks + 8 * lh) * 2);
 #pragma unroll
         for (int t = 0; t < QT; ++t)  // the first step takes rel_w / sm_scale as its accumulator input
-          s[t][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[t][ks], ks == 0 ? b1[t][nt] : s[t][nt], 0, 0, 0);
+          s[t][nt] = T::mfma(av, qf[t][ks], ks == 0 ? b1[t][nt] : s[t][nt]);
       }
     }
 
@@ -384,7 +412,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
     vt_issue(v_stage, integral_constant<int, 1>{}, vf[1]);
 
     // online softmax, one query per lane
-    bf16x8 pk[QT][4];
+    u32x4 pk[QT][4];
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
       float mx = s[t][0][0];
@@ -420,7 +448,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
         }
       if (!C::ONES_ROW) l_i[t] = l_i[t] * alpha + lsum;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) pk[t][j] = cvt_bf16x8(s[t][j >> 1], 8 * (j & 1));
+      for (int j = 0; j < 4; ++j) pk[t][j] = cvt_x8<T>(s[t][j >> 1], 8 * (j & 1));
     }
 
     // O^T += V^T P^T, the V^T fragments of key step j+1 in flight under the MFMAs of step j
@@ -432,7 +460,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
           const u32x4 w = {f[2 * dt][0], f[2 * dt][1], f[2 * dt + 1][0], f[2 * dt + 1][1]};
 #pragma unroll
           for (int t = 0; t < QT; ++t)
-            oacc[t][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(w), pk[t][j], oacc[t][dt], 0, 0, 0);
+            oacc[t][dt] = T::mfma(w, pk[t][j], oacc[t][dt]);
         }
       };
       vt_wait(integral_constant<int, NF>{}, vf[0]);
@@ -473,8 +501,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void attn_global_ke
       for (int j = 0; j < 4; ++j) {
         const int d = 32 * dt + 8 * j + 4 * lh;
         if (d < HD) {
-          const u32x2 o = {pack_bf16x2(oacc[t][dt][4 * j] * inv, oacc[t][dt][4 * j + 1] * inv),
-                           pack_bf16x2(oacc[t][dt][4 * j + 2] * inv, oacc[t][dt][4 * j + 3] * inv)};
+          const u32x2 o = {T::pack2(oacc[t][dt][4 * j] * inv, oacc[t][dt][4 * j + 1] * inv),
+                           T::pack2(oacc[t][dt][4 * j + 2] * inv, oacc[t][dt][4 * j + 3] * inv)};
           *reinterpret_cast<u32x2*>(op + d) = o;
         }
       }
@@ -515,20 +543,21 @@ struct WindowCfg {
   static_assert(NT <= WAVES, "one query tile per wavefront");
 };
 
-// one-hot bf16x8: element e is 1.0 iff slot == 8*lh + e
-SF_DEVICE bf16x8 onehot_bf16x8(int slot, int lh) {
+// one-hot vector of eight 16-bit elements: element e is 1.0 iff slot == 8*lh + e
+template <typename T>
+SF_DEVICE u32x4 onehot_x8(int slot, int lh) {
   const int e = slot - 8 * lh;  // may be outside [0, 8)
   u32x4 w;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     unsigned int v = 0u;
-    if ((e >> 1) == i) v = (e & 1) ? 0x3F800000u : 0x00003F80u;
+    if ((e >> 1) == i) v = (e & 1) ? (T::kOne << 16) : T::kOne;
     w[i] = v;
   }
-  return as_bf16x8(w);
+  return w;
 }
 
-template <int HD, bool FUSED>
+template <typename T, int HD, bool FUSED>
 __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(AttnArgs a) {
   using C = WindowCfg<HD>;
   __shared__ __attribute__((aligned(16))) unsigned char lds[C::LDS_BYTES];
@@ -577,22 +606,22 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
   const int qc = min(qi, N - 1);
 
   // ---- requests first: this wavefront's query rows, then the K / V staging loads ----------
-  bf16x8 qf[C::KS];
+  u32x4 qf[C::KS];
   {
     const unsigned short* qp = qbase + (int64_t)max(tok_of(qc), 0) * a.q_sn + 8 * lh;  // padding queries: any row
 #pragma unroll
-    for (int s = 0; s < C::KS; ++s) qf[s] = load_bf16x8_global(qp + 16 * s);
+    for (int s = 0; s < C::KS; ++s) qf[s] = load_x8_global(qp + 16 * s);
   }
   // the table rows both bias products need (row min(lr, 2g-2) of rel_pos_h and of rel_pos_w):
   // requested now, so that their latency runs under the K requests below
-  bf16x8 tfrag[FUSED ? 2 : 1][C::KS];
+  u32x4 tfrag[FUSED ? 2 : 1][C::KS];
   if (FUSED && has_tile) {
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
       const unsigned short* tab = which ? a.rw : a.rh;
       const int trow = min(lr, 2 * (which ? a.gw : a.gh) - 2);
 #pragma unroll
-      for (int s = 0; s < C::KS; ++s) tfrag[which][s] = load_bf16x8_global(tab + trow * HD + 16 * s + 8 * lh);
+      for (int s = 0; s < C::KS; ++s) tfrag[which][s] = load_x8_global(tab + trow * HD + 16 * s + 8 * lh);
     }
   }
   // wave instruction i of the window fills pieces 64i .. 64i+63: piece P is key P / PPR,
@@ -657,7 +686,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
         for (int r = 0; r < 16; ++r) tacc[r] = 0.f;
         if (has_tile) {
 #pragma unroll
-          for (int s = 0; s < C::KS; ++s) tacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tfrag[which][s], qf[s], tacc, 0, 0, 0);
+          for (int s = 0; s < C::KS; ++s) tacc = T::mfma(tfrag[which][s], qf[s], tacc);
         }
 #pragma unroll
         // stored in reverse (position 31 - rel), so that the lane's eight slots 8lh .. 8lh+7, which
@@ -665,7 +694,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
         for (int r = 0; r < 16; r += 2) {  // registers r, r+1 are adjacent rel: one packed 4-byte write
           const int rel = 8 * (r >> 2) + 4 * lh + (r & 3);
           *reinterpret_cast<unsigned int*>(X + lr * C::XSTR + 30 - rel) =
-              pack_bf16x2(tacc[r + 1] * a.inv_scale, tacc[r] * a.inv_scale);
+              T::pack2(tacc[r + 1] * a.inv_scale, tacc[r] * a.inv_scale);
         }
         wave_lds_fence();
         {
@@ -694,16 +723,16 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
 #pragma unroll
         for (int v = 0; v < 2; ++v) {
           const int slot = 8 * lh + 2 * i + v;
-          const float rh_raw = bf16_bits_to_f32(rhp[min(slot, a.gh - 1)]) * a.inv_scale;
-          const float rw_raw = bf16_bits_to_f32(rwp[min(slot, a.gw - 1)]) * a.inv_scale;
+          const float rh_raw = T::from_bits(rhp[min(slot, a.gh - 1)]) * a.inv_scale;
+          const float rw_raw = T::from_bits(rwp[min(slot, a.gw - 1)]) * a.inv_scale;
           fh[v] = (slot < a.gh) ? rh_raw : 0.f;
           fw[v] = (slot < a.gw) ? rw_raw : 0.f;
         }
-        bhw[i] = pack_bf16x2(fh[0], fh[1]);
-        bww[i] = pack_bf16x2(fw[0], fw[1]);
+        bhw[i] = T::pack2(fh[0], fh[1]);
+        bww[i] = T::pack2(fw[0], fw[1]);
       }
     }
-    if (lh == 1) bhw[3] = (bhw[3] & 0xffffu) | 0xF1490000u;  // slot 15 = -1e30 (bf16 0xF149)
+    if (lh == 1) bhw[3] = (bhw[3] & 0xffffu) | (T::kMask << 16);  // slot 15: the masking value
     const u32x4 bhv = {bhw[0], bhw[1], bhw[2], bhw[3]};
     const u32x4 bwv = {bww[0], bww[1], bww[2], bww[3]};
     bias_hv = bhv;
@@ -719,7 +748,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     *reinterpret_cast<u32x4*>(vl + (row * C::VSTR + col * 8) * 2) = z;
   }
   if (C::ONES_ROW && tid < 16 * nsteps) {  // the ones channel (P = 0 beyond the last key anyway)
-    const u32x4 one = {0x3F80u, 0u, 0u, 0u};
+    const u32x4 one = {T::kOne, 0u, 0u, 0u};
     *reinterpret_cast<u32x4*>(vl + (tid * C::VSTR + HD) * 2) = one;
   }
   if (!has_tile) {  // a wavefront without a query tile only helps with the staging and with the output
@@ -751,10 +780,10 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)p));
     const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)(p + 8 * C::VSTR * 2)));
     const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
-    return as_bf16x8(w);
+    return w;
   };
 
-  const bf16x8 bh_op = as_bf16x8(bias_hv), bw_op = as_bf16x8(bias_wv);
+  const u32x4 bh_op = bias_hv, bw_op = bias_wv;
 
   // ---- online softmax over the key tiles: S^T tile, running max, P, O^T += V^T P^T --------
   f32x16 oacc[C::DT];
@@ -773,15 +802,14 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
       for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < C::KS; ++ks) {
-        const bf16x8 av = as_bf16x8(
-            *reinterpret_cast<const u32x4*>(kl + (nc * C::KSTR + 16 * ks + 8 * lh) * 2));
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, qf[ks], acc, 0, 0, 0);
+        const u32x4 av = *reinterpret_cast<const u32x4*>(kl + (nc * C::KSTR + 16 * ks + 8 * lh) * 2);
+        acc = T::mfma(av, qf[ks], acc);
       }
       const int nh = div_gw(min(n, 255));
-      const bf16x8 ih = onehot_bf16x8(n < N ? nh : 15, lh);
-      const bf16x8 iw = onehot_bf16x8(n < N ? n - nh * a.gw : 99, lh);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ih, bh_op, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(iw, bw_op, acc, 0, 0, 0);
+      const u32x4 ih = onehot_x8<T>(n < N ? nh : 15, lh);
+      const u32x4 iw = onehot_x8<T>(n < N ? n - nh * a.gw : 99, lh);
+      acc = T::mfma(ih, bh_op, acc);
+      acc = T::mfma(iw, bw_op, acc);
 
       float mx = acc[0];
 #pragma unroll
@@ -817,10 +845,10 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
       for (int half = 0; half < 2; ++half) {
         const int j = 2 * nt + half;
         if (j < nsteps) {  // uniform
-          const bf16x8 pk = cvt_bf16x8(acc, 8 * half);
+          const u32x4 pk = cvt_x8<T>(acc, 8 * half);
 #pragma unroll
           for (int dt = 0; dt < C::DT; ++dt) {
-            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt_frag(dt, j), pk, oacc[dt], 0, 0, 0);
+            oacc[dt] = T::mfma(vt_frag(dt, j), pk, oacc[dt]);
           }
         }
       }
@@ -852,8 +880,8 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
       for (int j = 0; j < 4; ++j) {
         const int d = 32 * dt + 8 * j + 4 * lh;
         if (d < HD) {
-          const u32x2 o = {pack_bf16x2(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
-                           pack_bf16x2(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
+          const u32x2 o = {T::pack2(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
+                           T::pack2(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
           *reinterpret_cast<u32x2*>(orow_l + d * 2) = o;
         }
       }
@@ -881,7 +909,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
 // =============================================================================
 // host side
 // =============================================================================
-template <int HD, bool FUSED>
+template <typename T, int HD, bool FUSED>
 static int launch_hd(const AttnArgs& a, bool global_path, hipStream_t stream) {
   if (global_path) {
     constexpr int QT = 1;
@@ -890,7 +918,7 @@ static int launch_hd(const AttnArgs& a, bool global_path, hipStream_t stream) {
       using C = GlobalCfg<HD, QT, WAVES>;
       const int64_t total = (int64_t)a.B * a.nH * (a.N / C::BM);
       const unsigned int grid = (unsigned int)(((total + 7) / 8) * 8);
-      hipLaunchKernelGGL((attn_global_kernel<HD, QT, FUSED, WAVES>), dim3(grid), dim3(64 * WAVES), 0, stream, a);
+      hipLaunchKernelGGL((attn_global_kernel<T, HD, QT, FUSED, WAVES>), dim3(grid), dim3(64 * WAVES), 0, stream, a);
     };
     // 256 queries per workgroup when that still gives every CU several workgroups
     // (SAMFAST_ATTN_WAVES=4 / 8 overrides the choice where the shape allows it)
@@ -903,7 +931,7 @@ static int launch_hd(const AttnArgs& a, bool global_path, hipStream_t stream) {
   }
   const int64_t wins = a.ws > 0 ? (int64_t)a.B * a.wins_x * a.wins_y : a.B;
   const unsigned int grid = (unsigned int)(((wins * a.nH + 7) / 8) * 8);
-  hipLaunchKernelGGL((attn_window_kernel<HD, FUSED>), dim3(grid), dim3(WindowCfg<HD>::THREADS), 0, stream, a);
+  hipLaunchKernelGGL((attn_window_kernel<T, HD, FUSED>), dim3(grid), dim3(WindowCfg<HD>::THREADS), 0, stream, a);
   return check_launch("attn_window_kernel");
 }
 
@@ -913,7 +941,8 @@ static int attn_dispatch(bool fused, AttnArgs& a, int hd, int dtype, float sm_sc
   SF_REQUIRE(sm_scale > 0.f, "attn_relpos: sm_scale must be positive");
   // an empty batch is a valid call that does nothing (its buffers may be null)
   SF_REQUIRE(a.B == 0 || (a.q && a.k && a.v && a.out && a.rh && a.rw), "attn_relpos: null pointer");
-  if (dtype != SAMFAST_BF16) SF_FAIL(SAMFAST_E_UNSUPPORTED, "attn_relpos: only bf16 is built");
+  if (dtype != SAMFAST_BF16 && dtype != SAMFAST_F16)
+    SF_FAIL(SAMFAST_E_UNSUPPORTED, "attn_relpos: element type %d is neither SAMFAST_BF16 nor SAMFAST_F16", dtype);
   if (hd != 64 && hd != 80)
     SF_FAIL(SAMFAST_E_UNSUPPORTED, "attn_relpos: head_dim %d not in {64, 80}", hd);
   SF_REQUIRE((int64_t)a.B * a.nH < (1ll << 24), "attn_relpos: B*nH too large");
@@ -959,9 +988,13 @@ static int attn_dispatch(bool fused, AttnArgs& a, int hd, int dtype, float sm_sc
   if (a.B == 0) return SAMFAST_OK;
   a.c = sm_scale * kLog2e;
   a.inv_scale = 1.0f / sm_scale;
-  if (hd == 64)
-    return fused ? launch_hd<64, true>(a, global_path, stream) : launch_hd<64, false>(a, global_path, stream);
-  return fused ? launch_hd<80, true>(a, global_path, stream) : launch_hd<80, false>(a, global_path, stream);
+  auto by_type = [&](auto elem) {
+    using T = decltype(elem);
+    if (hd == 64)
+      return fused ? launch_hd<T, 64, true>(a, global_path, stream) : launch_hd<T, 64, false>(a, global_path, stream);
+    return fused ? launch_hd<T, 80, true>(a, global_path, stream) : launch_hd<T, 80, false>(a, global_path, stream);
+  };
+  return dtype == SAMFAST_F16 ? by_type(ElemF16{}) : by_type(ElemBf16{});
 }
 
 }  // namespace samfast

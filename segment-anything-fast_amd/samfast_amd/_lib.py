@@ -13,6 +13,7 @@ _LIB_PATH = Path(__file__).resolve().parent / "lib" / "libsamfast.so"
 _lib = None
 
 SAMFAST_BF16 = 0
+SAMFAST_F16 = 1  # attention entry points only
 
 _i32, _i64, _f32, _ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 

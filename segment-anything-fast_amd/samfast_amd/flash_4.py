@@ -14,8 +14,8 @@ natively (no pad to 128, :358-367), batch size 1 with head_dim 64 is correct
 (:350-351 disables it there), and 14x14 windows go to the HIP kernel as well
 (the reference sends them to SDPA with a materialised bias, :368-370).
 
-As in the reference, inputs the kernels do not cover (fp32, CPU tensors, the
-switch set to 0, odd shapes) take the eager
+Both half types run on the kernels (fp16 and bf16, :188,:348).  As in the reference, inputs the
+kernels do not cover (fp32, CPU tensors, the switch set to 0, odd shapes) take the eager
 F.scaled_dot_product_attention(attn_mask=rel_h + rel_w) route (:368-370); a GPU
 half-precision call that the kernels DO cover never falls back - a missing or
 failing library raises.
@@ -77,7 +77,8 @@ if _OWNS_SCHEMA:
 
 
 def _kernel_guards(q_, k_, v_) -> bool:
-    return (q_.is_cuda and q_.dtype == torch.bfloat16 and q_.dtype == k_.dtype
+    # half types only, as flash_4.py:345-348
+    return (q_.is_cuda and q_.dtype in (torch.bfloat16, torch.float16) and q_.dtype == k_.dtype
             and k_.dtype == v_.dtype and USE_CUSTOM_KERNEL)
 
 

@@ -77,9 +77,13 @@ def _bnhd_strides(t: torch.Tensor) -> Tuple[int, int, int]:
 
 
 def _dtype_code(t: torch.Tensor) -> int:
+    """Element type code of the C ABI.  The attention kernels exist for both half types; the
+    int8 linears take bfloat16 only and refuse the float16 code themselves."""
     if t.dtype == torch.bfloat16:
         return _lib.SAMFAST_BF16
-    raise RuntimeError(f"samfast: unsupported dtype {t.dtype} (the kernels are built for bfloat16)")
+    if t.dtype == torch.float16:
+        return _lib.SAMFAST_F16
+    raise RuntimeError(f"samfast: unsupported dtype {t.dtype} (the kernels take bfloat16 or float16)")
 
 
 def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: Optional[torch.Tensor],
@@ -99,7 +103,7 @@ def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: Optional[
 def attn_supported(N: int, grid_hw: Tuple[int, int], hd: int, dtype: torch.dtype) -> bool:
     """Shapes the HIP attention kernels cover (mirrors the checks in the library)."""
     gh, gw = grid_hw
-    if dtype != torch.bfloat16 or hd not in (64, 80) or gh * gw != N:
+    if dtype not in (torch.bfloat16, torch.float16) or hd not in (64, 80) or gh * gw != N:
         return False
     global_ok = gw == 64 and N % 128 == 0 and gh <= 64
     window_ok = gh <= 15 and gw <= 16 and N <= 208

@@ -85,8 +85,10 @@ def test_argument_validation_without_gpu():
     assert rc == -2 and b"head_dim" in lib.samfast_last_error()
     rc = lib.samfast_attn_relpos_fwd(p, p, p, p, p, p, 1, 1, 20, 20, 64, *([64] * 12), 0, 0.125, None)
     assert rc == -2 and b"neither" in lib.samfast_last_error()
-    rc = lib.samfast_attn_relpos_fwd(p, p, p, p, p, p, 1, 1, 14, 14, 64, *([64] * 12), 1, 0.125, None)
-    assert rc == -2  # any element type other than SAMFAST_BF16
+    rc = lib.samfast_attn_relpos_fwd(p, p, p, p, p, p, 1, 1, 14, 14, 64, *([64] * 12), 2, 0.125, None)
+    assert rc == -2 and b"element type" in lib.samfast_last_error()  # neither SAMFAST_BF16 nor SAMFAST_F16
+    rc = lib.samfast_quant_rowwise_i8(p, 64, p, p, 4, 64, 1, 0, None)
+    assert rc == -2  # the linears are bf16 only
 
 
 def test_ops_refuse_cpu_tensors():

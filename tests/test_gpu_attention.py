@@ -225,15 +225,16 @@ def test_global_kernel_wave_count_variants_agree(monkeypatch, hd, gh):
 
 @pytest.mark.parametrize("batch", [1, 8])
 @pytest.mark.parametrize("head,hidden_dim", [(16, 80), (12, 64)])
-def test_reference_test_recipe_against_sdpa(batch, head, hidden_dim):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_reference_test_recipe_against_sdpa(batch, head, hidden_dim, dtype):
     """The reference's own test of this operator (test/test_flash_4.py:5-43): its shapes (batch 1
-    and 8, 16 heads x 80 / 12 heads x 64, 4096 tokens), its input recipe (seed 20, q / k / v and
-    both bias factors ~ N(0, 0.5)) and its tolerance (rtol = atol = 1e-3) against
-    scaled_dot_product_attention with the materialised bias, here for the dtype the kernels are
-    built for (bf16); SDPA is evaluated in fp32 on the same bf16 inputs and rounded once."""
+    and 8, 16 heads x 80 / 12 heads x 64, 4096 tokens), its two dtypes (:41-43), its input recipe
+    (seed 20, q / k / v and both bias factors ~ N(0, 0.5)) and its tolerance (rtol = atol = 1e-3)
+    against scaled_dot_product_attention with the materialised bias; SDPA is evaluated in fp32 on
+    the same half-precision inputs and rounded once."""
     from samfast_amd.flash_4 import _attention_rel_h_rel_w
-    seq_len, dtype, device = 4096, torch.bfloat16, "cuda"
-    print(f"case reference recipe batch={batch} head={head} hd={hidden_dim}", flush=True)
+    seq_len, device = 4096, "cuda"
+    print(f"case reference recipe batch={batch} head={head} hd={hidden_dim} {dtype}", flush=True)
     torch.manual_seed(20)
     q, k, v = (torch.empty((batch, head, seq_len, hidden_dim), dtype=dtype, device=device).normal_(mean=0.0, std=0.5)
                for _ in range(3))
@@ -269,3 +270,71 @@ def test_seeded_sweep_of_window_and_grid_shapes():
         out = ops.attn_relpos(q.cuda(), k.cuda(), v.cuda(), rph.cuda(), rpw.cuda(), (gh, gw))
         torch.cuda.synchronize()
         _check(out, ref, f"sweep {B}x{nH}x{gh}x{gw}x{hd}")
+
+
+@pytest.mark.parametrize("B,nH,gh,gw,hd", [(1, 2, 64, 64, 64), (2, 2, 64, 64, 80), (3, 2, 14, 14, 64),
+                                           (4, 3, 14, 14, 80), (2, 2, 7, 9, 80), (1, 1, 13, 16, 64)])
+def test_float16_operands_vs_oracle(B, nH, gh, gw, hd):
+    """The float16 instantiation of both kernels (the reference's operator takes fp16 and bf16,
+    flash_4.py:188,348): tables form and bias form against the fp32 oracle on the same
+    fp16-rounded inputs, at the bar of the bf16 tests."""
+    from samfast_amd import ops
+    print(f"case fp16 B={B} nH={nH} grid={gh}x{gw} hd={hd}", flush=True)
+    q, k, v, rph, rpw = attn_inputs(B, nH, gh, gw, hd, dtype=torch.float16)
+    ref = _oracle_tables(q, k, v, rph, rpw, (gh, gw))
+    out = ops.attn_relpos(q.cuda(), k.cuda(), v.cuda(), rph.cuda(), rpw.cuda(), (gh, gw))
+    assert out.dtype == torch.float16
+    _check(out, ref, f"fp16 fused {B}x{nH}x{gh}x{gw}x{hd}")
+    q, k, v, rel_h, rel_w = bias_inputs(B, nH, gh, gw, hd, dtype=torch.float16)
+    ref = ora.attention_rel_h_rel_w(q, k, v, rel_h, rel_w, compute_dtype=torch.float32)
+    out = ops.attn_relpos_bias(q.cuda(), k.cuda(), v.cuda(), rel_h.squeeze(-1).cuda(), rel_w.squeeze(-2).cuda())
+    _check(out, ref, f"fp16 bias {B}x{nH}x{gh}x{gw}x{hd}")
+
+
+def test_float16_windowed_on_image_tokens_and_module():
+    """fp16 through the image-ordered window entry point (padding rows included) against the oracle
+    on explicitly partitioned windows, and through the Attention module (fp16 nn.Linear + the HIP
+    kernel) against the module's eager route."""
+    from samfast_amd import flash_4, ops
+    from samfast_amd.modeling import Attention
+    B, nH, H, W, ws, hd = 2, 3, 20, 17, 14, 80
+    g = torch.Generator().manual_seed(5)
+    C = nH * hd
+    f16 = torch.float16
+    qkv = torch.randn((B, H * W, 3, nH, hd), generator=g).to(f16)
+    rph = (torch.randn((2 * ws - 1, hd), generator=g) * 0.02).to(f16)
+    rpw = (torch.randn((2 * ws - 1, hd), generator=g) * 0.02).to(f16)
+    pad_k, pad_v = torch.randn((nH, hd), generator=g).to(f16), torch.randn((nH, hd), generator=g).to(f16)
+    dq = qkv.cuda()
+    q, k, v = (dq[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    out = ops.attn_relpos_windowed(q, k, v, rph.cuda(), rpw.cuda(), pad_k.cuda(), pad_v.cuda(), (H, W), ws, hd ** -0.5)
+    Hp, Wp = -(-H // ws) * ws, -(-W // ws) * ws
+
+    def part(t, fill):
+        full = fill.reshape(1, 1, 1, C).float().expand(B, Hp, Wp, C).clone()
+        full[:, :H, :W] = t.reshape(B, H, W, C).float()
+        wins, _ = ora.window_partition(full, ws)
+        return wins.reshape(-1, ws * ws, nH, hd).permute(0, 2, 1, 3).to(f16)
+    qw, kw, vw = part(qkv[:, :, 0], torch.zeros(C)), part(qkv[:, :, 1], pad_k), part(qkv[:, :, 2], pad_v)
+    ref = ora.attention_from_tables(qw, kw, vw, rph, rpw, (ws, ws))
+    ref = ref.permute(0, 2, 1, 3).reshape(-1, ws, ws, C).float()
+    ref = ora.window_unpartition(ref, ws, (Hp, Wp), (H, W)).reshape(B, H * W, nH, hd)
+    _check(out, ref, "fp16 windowed on image tokens")
+
+    torch.manual_seed(1)
+    att = Attention(256, 4, use_rel_pos=True, input_size=(14, 14))
+    with torch.no_grad():
+        att.rel_pos_h.normal_(0, 0.02)
+        att.rel_pos_w.normal_(0, 0.02)
+    att = att.eval().to(f16).cuda()
+    x = torch.randn(3, 14, 14, 256, device="cuda").to(f16)
+    with torch.no_grad():
+        got = att(x)
+        flash_4.USE_CUSTOM_KERNEL = False
+        try:
+            eager = att(x)
+        finally:
+            flash_4.USE_CUSTOM_KERNEL = True
+    assert got.dtype == f16
+    d = (got.float() - eager.float()).abs()
+    assert d.max().item() <= 2e-2 and d.mean().item() <= 1e-3, (d.max().item(), d.mean().item())
