@@ -54,6 +54,8 @@ def parse():
     p.add_argument("--batch", type=int, default=16)
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-gpu-baseline", action="store_true")
+    p.add_argument("--no-compiled-baseline", action="store_true",
+                   help="skip the torch.compile variant of the PyTorch-ROCm baseline (about 30 s)")
     p.add_argument("--main-only", action="store_true",
                    help="measure only the workload named by --model / --batch (no other_configs object)")
     p.add_argument("--no-mfma-ceiling", action="store_true", help="skip the matrix-instruction-only loops")
@@ -251,7 +253,8 @@ def mfma_ceiling():
 
 
 def run_config(model, batch, steps, warmup, sparse_mlp=False, bf16_linears=False, graph=False,
-               gpu_baseline=True, calibration_copy=False, yardsticks=False, also_graph=False):
+               gpu_baseline=True, calibration_copy=False, yardsticks=False, also_graph=False,
+               compiled_baseline=False):
     """Build the encoder, time `steps` forwards after `warmup`, run one instrumented forward for the
     per-kernel figures and (optionally) the PyTorch-ROCm eager baseline on the same weights."""
     import torch
@@ -357,6 +360,20 @@ def run_config(model, batch, steps, warmup, sparse_mlp=False, bf16_linears=False
                 ref = base(images)
             cos = torch.nn.functional.cosine_similarity(
                 out.float().flatten(1), ref.float().flatten(1), dim=1).min().item()
+            compiled = None
+            if compiled_baseline:
+                # the reference's "SDPA" configuration is this eager model under torch.compile
+                # (build_sam.py:67-71); default mode: no autotuning, ~20 s of compilation
+                try:
+                    cbase = torch.compile(base)
+                    with torch.no_grad():
+                        csec = time_steps(lambda: cbase(images), 3, 2)
+                    compiled = {"what": "the same model under torch.compile (default mode)",
+                                "value": round(batch / csec, 3), "unit": "images/s",
+                                "ms_per_step": round(csec * 1e3, 3), "speedup": round(csec / sec, 3)}
+                    del cbase
+                except Exception as e:  # the baseline is optional: a compiler problem must not lose the line
+                    compiled = {"what": "torch.compile failed", "error": f"{type(e).__name__}: {str(e)[:200]}"}
         finally:
             flash_4.USE_CUSTOM_KERNEL = True
         result["gpu_baseline"] = {"what": "same encoder, PyTorch-ROCm eager bf16 SDPA(attn_mask) + bf16 nn.Linear",
@@ -364,6 +381,8 @@ def run_config(model, batch, steps, warmup, sparse_mlp=False, bf16_linears=False
                                   "ms_per_step": round(bsec * 1e3, 3),
                                   "speedup": round(bsec / sec, 3),
                                   "min_cosine_vs_this_path": round(cos, 6)}
+        if compiled is not None:
+            result["gpu_baseline"]["torch_compile"] = compiled
         del base, ref
 
     if yardsticks:
@@ -413,7 +432,8 @@ def main():
     main_run, sd_fp32 = run_config(
         args.model, args.batch, args.steps, args.warmup, sparse_mlp=args.sparse_mlp,
         bf16_linears=args.bf16_linears, graph=args.graph, gpu_baseline=not args.no_gpu_baseline,
-        calibration_copy=args.calibration_copy, yardsticks=args.library_yardsticks)
+        calibration_copy=args.calibration_copy, yardsticks=args.library_yardsticks,
+        compiled_baseline=not args.no_gpu_baseline and not args.no_compiled_baseline)
 
     result = {
         "metric": ("images/s ViT-H encoder bs16 1024^2" if (args.model, args.batch) == ("vit_h", 16)
