@@ -341,7 +341,7 @@ SF_DEVICE void gemm_quant_tail(const GemmArgs& a, int m0, int tile_m, int tid, i
   q.xq = a.yq; q.sx = a.sy; q.M = a.M; q.K = TAILN;
   q.eps = a.ln_eps; q.inv_K = 1.0f / (float)TAILN; q.kb64 = a.yq_kb64;
   constexpr int nchunk = TAILN / EPC;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: rows and their addresses stay scalar
   typename RQ::in_t gw[NCH], bw[NCH];
   if (TAILLN) RQ::load_affine(q.gamma, q.beta, nchunk, lane, gw, bw);
   // wavefront w takes rows w, w + 4, ...; the loads of the next DEPTH - 1 rows are in flight while

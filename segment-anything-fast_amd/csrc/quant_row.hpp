@@ -135,12 +135,21 @@ struct RowQuantizer {
   }
 
   // chunk c of output row `row`: row-major at row*K + EPC*c; K-block major at
-  // ((c*EPC/64)*M + row)*64 + (c*EPC)%64
+  // ((c*EPC/64)*M + row)*64 + (c*EPC)%64.  Written as a uniform base (the row is the same for the
+  // whole wavefront) plus an unsigned 32-bit lane offset - M*K < 2^31 is checked on the host - so
+  // that the stores take the scalar-base form and no 64-bit arithmetic runs per lane.
   static SF_DEVICE void store_chunk(const QuantArgs& a, int64_t row, int c, const unsigned int (&codes)[EPC / 4]) {
-    const int k = c * EPC;
-    const int64_t off = a.kb64 ? ((int64_t)(k >> 6) * a.M + row) * 64 + (k & 63)
-                               : row * (int64_t)a.K + k;
-    unsigned int* dst = reinterpret_cast<unsigned int*>(a.xq + off);
+    const unsigned int k = (unsigned int)c * EPC;
+    int8_t* base;
+    unsigned int off;
+    if (a.kb64) {
+      base = a.xq + row * 64;
+      off = (k >> 6) * ((unsigned int)a.M * 64u) + (k & 63u);
+    } else {
+      base = a.xq + row * (int64_t)a.K;
+      off = k;
+    }
+    unsigned int* dst = reinterpret_cast<unsigned int*>(base + off);
     if (EPC == 8) {
       const u32x2 o = {codes[0], codes[EPC / 4 - 1]};
       *reinterpret_cast<u32x2*>(dst) = o;

@@ -24,7 +24,9 @@ template <int NCH, int EPC, bool LN>
 __global__ __launch_bounds__(64 * kQuantWavesPerBlock) void quant_rowwise_bf16_kernel(QuantArgs a) {
   using RQ = RowQuantizer<NCH, EPC, LN>;
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * kQuantWavesPerBlock + (threadIdx.x >> 6);
+  // the wavefront index is uniform: telling the compiler so keeps the row and everything derived from it
+  // (row pointers, output offsets) in scalar registers instead of 64-bit arithmetic per lane
+  const int64_t row = (int64_t)blockIdx.x * kQuantWavesPerBlock + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   if (row >= a.M) return;  // whole wavefront leaves together
   const int nchunk = a.K / EPC;
 
@@ -82,6 +84,7 @@ static int check_common(const char* who, const void* x, int64_t ldx, const int8_
   SF_REQUIRE(aligned16(x) && (reinterpret_cast<uintptr_t>(xq) & 7u) == 0,
              "%s: x must be 16-byte and xq 8-byte aligned", who);
   SF_REQUIRE((M + 3) / 4 < (1ll << 31), "%s: M too large", who);
+  SF_REQUIRE(M * (int64_t)K < (1ll << 31), "%s: outputs of 2 GiB or more are not supported (the GEMM cannot read them)", who);
   return SAMFAST_OK;
 }
 
