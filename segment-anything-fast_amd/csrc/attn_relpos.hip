@@ -757,137 +757,136 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
   }
 
   if (has_tile) {
-  // V^T operand through transposing LDS reads (ds_read_b64_tr_b16): in each group of 16 lanes,
-  // lane l receives as element j the l%4-th 16-bit value of the 8 bytes addressed by lane
-  // 4j + l/4.  Source lane 4j + i points at key j of the lane half's four keys, channels
-  // 4i .. 4i+3 of the group's 16 channels; lane l ends up with channel l of four keys.
-  int vrd[C::DT];
-  {
-    const int g = lane >> 4, sl = lane & 15;
-    const int key = 4 * (g >> 1) + (sl >> 2);
+    // V^T operand through transposing LDS reads (ds_read_b64_tr_b16): in each group of 16 lanes,
+    // lane l receives as element j the l%4-th 16-bit value of the 8 bytes addressed by lane
+    // 4j + l/4.  Source lane 4j + i points at key j of the lane half's four keys, channels
+    // 4i .. 4i+3 of the group's 16 channels; lane l ends up with channel l of four keys.
+    int vrd[C::DT];
+    {
+      const int g = lane >> 4, sl = lane & 15;
+      const int key = 4 * (g >> 1) + (sl >> 2);
 #pragma unroll
-    for (int dt = 0; dt < C::DT; ++dt) {
-      int d = 32 * dt + 16 * (g & 1) + 4 * (sl & 3);
-      if (C::ONES_ROW) d = d >= HD + 8 ? HD + 4 : d;  // past the spare piece (1, 0, .., 0): its zero half
-      else d = min(d, HD - 4);
-      vrd[dt] = (key * C::VSTR + d) * 2;
+      for (int dt = 0; dt < C::DT; ++dt) {
+        int d = 32 * dt + 16 * (g & 1) + 4 * (sl & 3);
+        if (C::ONES_ROW) d = d >= HD + 8 ? HD + 4 : d;  // past the spare piece (1, 0, .., 0): its zero half
+        else d = min(d, HD - 4);
+        vrd[dt] = (key * C::VSTR + d) * 2;
+      }
     }
-  }
-  auto vt_frag = [&](int dt, int j) {
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    typedef __attribute__((address_space(3))) s16x4* trptr_t;
-    const unsigned char* p = vl + vrd[dt] + 16 * j * C::VSTR * 2;
-    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)p));
-    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)(p + 8 * C::VSTR * 2)));
-    const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
-    return w;
-  };
+    auto vt_frag = [&](int dt, int j) {
+      typedef short s16x4 __attribute__((ext_vector_type(4)));
+      typedef __attribute__((address_space(3))) s16x4* trptr_t;
+      const unsigned char* p = vl + vrd[dt] + 16 * j * C::VSTR * 2;
+      const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)p));
+      const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)(p + 8 * C::VSTR * 2)));
+      const u32x4 w = {lo[0], lo[1], hi[0], hi[1]};
+      return w;
+    };
 
-  const u32x4 bh_op = bias_hv, bw_op = bias_wv;
+    const u32x4 bh_op = bias_hv, bw_op = bias_wv;
 
-  // ---- online softmax over the key tiles: S^T tile, running max, P, O^T += V^T P^T --------
-  f32x16 oacc[C::DT];
+    // ---- online softmax over the key tiles: S^T tile, running max, P, O^T += V^T P^T --------
+    f32x16 oacc[C::DT];
 #pragma unroll
-  for (int dt = 0; dt < C::DT; ++dt)
+    for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
-  float m_run = -3.0e38f, l_run = 0.f;
+      for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+    float m_run = -3.0e38f, l_run = 0.f;
 #pragma unroll
-  for (int nt = 0; nt < C::NT; ++nt) {
-    if (32 * nt < N) {  // uniform
-      const int n = 32 * nt + lr;
-      const int nc = min(n, N - 1);
-      f32x16 acc;
+    for (int nt = 0; nt < C::NT; ++nt) {
+      if (32 * nt < N) {  // uniform
+        const int n = 32 * nt + lr;
+        const int nc = min(n, N - 1);
+        f32x16 acc;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < C::KS; ++ks) {
-        const u32x4 av = *reinterpret_cast<const u32x4*>(kl + (nc * C::KSTR + 16 * ks + 8 * lh) * 2);
-        acc = T::mfma(av, qf[ks], acc);
-      }
-      const int nh = div_gw(min(n, 255));
-      const u32x4 ih = onehot_x8<T>(n < N ? nh : 15, lh);
-      const u32x4 iw = onehot_x8<T>(n < N ? n - nh * a.gw : 99, lh);
-      acc = T::mfma(ih, bh_op, acc);
-      acc = T::mfma(iw, bw_op, acc);
+        for (int ks = 0; ks < C::KS; ++ks) {
+          const u32x4 av = *reinterpret_cast<const u32x4*>(kl + (nc * C::KSTR + 16 * ks + 8 * lh) * 2);
+          acc = T::mfma(av, qf[ks], acc);
+        }
+        const int nh = div_gw(min(n, 255));
+        const u32x4 ih = onehot_x8<T>(n < N ? nh : 15, lh);
+        const u32x4 iw = onehot_x8<T>(n < N ? n - nh * a.gw : 99, lh);
+        acc = T::mfma(ih, bh_op, acc);
+        acc = T::mfma(iw, bw_op, acc);
 
-      float mx = acc[0];
+        float mx = acc[0];
 #pragma unroll
-      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, acc[r]);
-      mx = max_with_lane_xor32(mx);
-      // lazy reference (see the global kernel): m_run follows the maximum in steps > 2^kLazyLog2
-      const float m_new = fmaxf(m_run, mx);
-      float alpha = 1.0f;
-      const bool move = __any((m_new - m_run) * a.c > kLazyLog2);  // uniform; first tile: always
-      if (move) {
-        alpha = fast_exp2((m_run - m_new) * a.c);
-        m_run = m_new;
-      }
-      const float neg_m = -m_run * a.c;
-      float lsum = 0.f;
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, acc[r]);
+        mx = max_with_lane_xor32(mx);
+        // lazy reference (see the global kernel): m_run follows the maximum in steps > 2^kLazyLog2
+        const float m_new = fmaxf(m_run, mx);
+        float alpha = 1.0f;
+        const bool move = __any((m_new - m_run) * a.c > kLazyLog2);  // uniform; first tile: always
+        if (move) {
+          alpha = fast_exp2((m_run - m_new) * a.c);
+          m_run = m_new;
+        }
+        const float neg_m = -m_run * a.c;
+        float lsum = 0.f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = fast_exp2(fmaf(acc[r], a.c, neg_m));
-        acc[r] = p;
-        if (!C::ONES_ROW) lsum += p;
-      }
-      if (!C::ONES_ROW) l_run = l_run * alpha + lsum;
-      if (nt == 0) {  // V travelled under the first score tile; every wavefront's share has landed
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-      } else if (move) {
+        for (int r = 0; r < 16; ++r) {
+          const float p = fast_exp2(fmaf(acc[r], a.c, neg_m));
+          acc[r] = p;
+          if (!C::ONES_ROW) lsum += p;
+        }
+        if (!C::ONES_ROW) l_run = l_run * alpha + lsum;
+        if (nt == 0) {  // V travelled under the first score tile; every wavefront's share has landed
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          __syncthreads();
+        } else if (move) {
 #pragma unroll
-        for (int dt = 0; dt < C::DT; ++dt)
+          for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-      }
+            for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+        }
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int j = 2 * nt + half;
-        if (j < nsteps) {  // uniform
-          const u32x4 pk = cvt_x8<T>(acc, 8 * half);
+        for (int half = 0; half < 2; ++half) {
+          const int j = 2 * nt + half;
+          if (j < nsteps) {  // uniform
+            const u32x4 pk = cvt_x8<T>(acc, 8 * half);
 #pragma unroll
-          for (int dt = 0; dt < C::DT; ++dt) {
-            oacc[dt] = T::mfma(vt_frag(dt, j), pk, oacc[dt]);
+            for (int dt = 0; dt < C::DT; ++dt) {
+              oacc[dt] = T::mfma(vt_frag(dt, j), pk, oacc[dt]);
+            }
           }
         }
       }
     }
-  }
-  float l;
-  if (C::ONES_ROW) {
-    // output row HD = tile DT-1, row HD % 32, held by the lh = (HD % 32) / 4 % 2 lanes
-    constexpr int orow = HD % 32;
-    constexpr int oreg = 4 * (orow / 8) + orow % 4, olh = (orow / 4) % 2;
-    const float own = oacc[C::DT - 1][oreg];
-    const float other = xor32(own);
-    l = (lh == olh) ? own : other;
-  } else {
-    l = l_run + xor32(l_run);
-  }
-  const float inv = 1.0f / l;
-  // ---- output: through LDS, so that a token's HD channels leave as one contiguous run ----------
-  // Written straight from the accumulators a lane would store 8 bytes to each of 32 different
-  // token rows per instruction; staged as (token, channel) rows in the K area - free once every
-  // wavefront has left its key loop - the whole workgroup then writes 16 bytes per lane with the
-  // HD/8 pieces of a token in neighbouring lanes.
-  __syncthreads();
-  if (qi < N) {
-    unsigned char* orow_l = kl + qi * (C::KSTR * 2);
+    float l;
+    if (C::ONES_ROW) {
+      // output row HD = tile DT-1, row HD % 32, held by the lh = (HD % 32) / 4 % 2 lanes
+      constexpr int orow = HD % 32;
+      constexpr int oreg = 4 * (orow / 8) + orow % 4, olh = (orow / 4) % 2;
+      const float own = oacc[C::DT - 1][oreg];
+      const float other = xor32(own);
+      l = (lh == olh) ? own : other;
+    } else {
+      l = l_run + xor32(l_run);
+    }
+    const float inv = 1.0f / l;
+    // ---- output: through LDS, so that a token's HD channels leave as one contiguous run ----------
+    // Written straight from the accumulators a lane would store 8 bytes to each of 32 different
+    // token rows per instruction; staged as (token, channel) rows in the K area - free once every
+    // wavefront has left its key loop - the whole workgroup then writes 16 bytes per lane with the
+    // HD/8 pieces of a token in neighbouring lanes.
+    __syncthreads();
+    if (qi < N) {
+      unsigned char* orow_l = kl + qi * (C::KSTR * 2);
 #pragma unroll
-    for (int dt = 0; dt < C::DT; ++dt)
+      for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int d = 32 * dt + 8 * j + 4 * lh;
-        if (d < HD) {
-          const u32x2 o = {T::pack2(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
-                           T::pack2(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
-          *reinterpret_cast<u32x2*>(orow_l + d * 2) = o;
+        for (int j = 0; j < 4; ++j) {
+          const int d = 32 * dt + 8 * j + 4 * lh;
+          if (d < HD) {
+            const u32x2 o = {T::pack2(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
+                             T::pack2(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv)};
+            *reinterpret_cast<u32x2*>(orow_l + d * 2) = o;
+          }
         }
-      }
-  }
-  }  // has_tile
-  else {
+    }
+  } else {
     __syncthreads();  // the key loops are over: the K area becomes the output staging area
   }
   __syncthreads();    // the staged output is complete
