@@ -648,28 +648,47 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
 
 
 // =============================================================================================
-// Three workgroups per CU.  Same 128x256x64 tile, same LDS layout, same arithmetic as
-// gemm_i8_kernel<EPI, 2, false>; what changes is the budget: at most 168 registers per lane and
-// 53 KB of LDS per workgroup, so that a third workgroup fits on the CU.  While one workgroup is
-// in its epilogue (no matrix instructions for 7-16 K cycles), two others are in their loops and
-// keep the matrix pipe fed - with two resident workgroups the one left in its loop cannot.
-//   * operand fragments are single-buffered (24 registers): the other wavefronts of the SIMD
-//     cover a wavefront's LDS read latency;
+// Three (or more) workgroups per CU.  Same LDS layout and arithmetic as gemm_i8_kernel<EPI, 2,
+// false>; what changes is the budget: at most 168 registers per lane and 53 KB of LDS per
+// workgroup, so that a third workgroup fits on the CU.  While one workgroup is in its epilogue
+// (no matrix instructions for 7-16 K cycles), two others are in their loops.
+//   * operand fragments are single-buffered: the other wavefronts of the SIMD cover a
+//     wavefront's LDS read latency;
 //   * two LDS stages: at the top of iteration kt every wavefront has finished tile kt-1
 //     (barrier), so tile kt+1 is requested into the stage tile kt-1 used, and has the whole
 //     iteration to land;
-//   * the epilogue is staged through LDS in two halves of 64 rows (the full 128 x 256 bf16 tile
-//     does not fit in 48 KB), residual values are fetched after the conversion work.
+//   * the epilogue is staged through LDS 64 rows at a time (the full bf16 tile does not fit
+//     next to nothing in 48 KB), residual values are fetched after the conversion work.
+// The tile is BM x BN = 128 x 256 (waves 2 x 2, each 64 x 128: 2 x 4 MFMA tiles), or 64 x 128
+// (each wave 32 x 64: 1 x 2 tiles, 32 accumulators, 27 KB of LDS) for launches whose large tiles
+// would leave most of the GPU's workgroup slots empty (4096 rows of a single image): four times
+// the workgroups, each a quarter of the work.
 // =============================================================================================
-template <int EPI>
-__global__ __launch_bounds__(256, 3) void gemm_i8_kernel3(GemmArgs a) {
+template <int BM, int BN>
+struct Gemm3Cfg {
+  static constexpr int TMW = BM / 64, TNW = BN / 64;  // MFMA tiles per wavefront: rows, columns
+  static constexpr int NST = 2;
+  static constexpr int GSTAGE = (BM + BN) * GLD;
+  static constexpr int NLD = (BM + BN) / 64;          // global->LDS wave instructions per tile and wavefront
+  static constexpr int EP_PITCH = BN * 2 + 32;        // staged output tile: row pitch in bytes
+  static constexpr int SX_OFF = 0, SW_OFF = BM * 4, BIAS_OFF = SW_OFF + BN * 4, MAP_OFF = BIAS_OFF + BN * 4;
+  static constexpr int SC_BYTES = MAP_OFF + BM * 4;
+  static constexpr int LDS_BYTES = NST * GSTAGE + SC_BYTES;
+  static constexpr int CHUNKS = BN / 8;               // 16-byte pieces per output row
+  static constexpr int ROWS_PER_PASS = 256 / CHUNKS;  // output rows the workgroup stores per pass
+  static constexpr int PASSES = 64 / ROWS_PER_PASS;   // passes over a staged 64-row tile
+  static constexpr int MIN_WG = BM == 128 ? 3 : 4;
+  static_assert(64 * EP_PITCH <= NST * GSTAGE, "a 64-row output tile must fit in the operand stages");
+  static_assert((BM == 128 && BN == 256) || (BM == 64 && BN == 128), "tile shapes built");
+};
+
+template <int EPI, int BM, int BN>
+__global__ __launch_bounds__(256, (Gemm3Cfg<BM, BN>::MIN_WG)) void gemm_i8_kernel3(GemmArgs a) {
   static_assert(EPI != EPI_I32, "bf16 epilogues only");
-  constexpr int GBM = 128, TM = 2, NST = 2;
-  constexpr int GSTAGE = (GBM + GBN) * GLD;  // 24 KB
-  constexpr int NLD = (GBM + GBN) / 64;      // global->LDS wave instructions per tile and wavefront: 6
-  static_assert(64 * EP_STRIDE <= NST * GSTAGE, "half an output tile must fit in the operand stages");
-  __shared__ __attribute__((aligned(16))) unsigned char lds[NST * GSTAGE + EP_SCALE_BYTES + EP_ROWMAP_BYTES];
-  unsigned char* sc = lds + NST * GSTAGE;
+  using C = Gemm3Cfg<BM, BN>;
+  constexpr int TMW = C::TMW, TNW = C::TNW, NLD = C::NLD, GSTAGE = C::GSTAGE;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[C::LDS_BYTES];
+  unsigned char* sc = lds + C::NST * GSTAGE;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -684,24 +703,26 @@ __global__ __launch_bounds__(256, 3) void gemm_i8_kernel3(GemmArgs a) {
   const unsigned int first_m = (pid / per_group) * a.group_m;
   const unsigned int gsz = min((unsigned int)a.tiles_m - first_m, (unsigned int)a.group_m);
   const unsigned int in_group = pid % per_group;
-  const int m0 = (int)(first_m + in_group % gsz) * GBM;
-  const int n0 = (int)(in_group / gsz) * GBN;
+  const int m0 = (int)(first_m + in_group % gsz) * BM;
+  const int n0 = (int)(in_group / gsz) * BN;
 
   typedef __attribute__((address_space(1))) const void* gptr_t;
   typedef __attribute__((address_space(3))) void* lptr_t;
 
-  // lane offsets of the six tile loads (see gemm_i8_kernel: swizzle applied to the global address,
-  // W rows permuted so that a lane ends with 4 adjacent output columns)
+  // lane offsets of the tile loads (see gemm_i8_kernel: the XOR swizzle is applied to the global
+  // address; W rows are permuted - slot s of a wavefront's BN/2 columns holds W row (s % 32) * TNW
+  // + s / 32 - so that a lane ends with TNW adjacent output columns)
   unsigned int dma_off[NLD];
 #pragma unroll
   for (int i = 0; i < NLD; ++i) {
     const int rho = 16 * (wave_u + 4 * i) + (lane >> 2);
     const int chunk = (lane & 3) ^ lds_swizzle(rho);
-    if (i < GBM / 64) {
+    if (i < BM / 64) {
       dma_off[i] = (unsigned int)(min(m0 + rho, a.M - 1) * a.row_pitch + chunk * 16);
     } else {
-      const int sl = rho - GBM;
-      const int wrow = (sl & 128) + (sl & 31) * 4 + ((sl & 127) >> 5);
+      const int sl = rho - BM;                      // slot inside the W part of the stage
+      const int half = sl / (BN / 2), sh = sl % (BN / 2);
+      const int wrow = half * (BN / 2) + (sh & 31) * TNW + (sh >> 5);
       dma_off[i] = (unsigned int)(min(n0 + wrow, a.N - 1) * a.row_pitch + chunk * 16);
     }
   }
@@ -713,36 +734,37 @@ __global__ __launch_bounds__(256, 3) void gemm_i8_kernel3(GemmArgs a) {
     for (int i = 0; i < NLD; ++i) {
       unsigned int off = dma_off[i];
       asm volatile("" : "+v"(off));
-      const int8_t* src = (i < GBM / 64 ? xb : wb) + off;
+      const int8_t* src = (i < BM / 64 ? xb : wb) + off;
       unsigned char* dst = lds + stage_off + (wave_u + 4 * i) * 1024;
       __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
     }
   };
 
   {
-    // row scales, column scales, bias (and row map) of this tile, 4 bytes per lane, straight into LDS
-    const int mm = min(m0 + (wave_u & 1) * 64 + lane, a.M - 1);
-    const int nn = min(n0 + wave_u * 64 + lane, a.N - 1);
-    __builtin_amdgcn_global_load_lds((gptr_t)(a.sx + mm), (lptr_t)(sc + (wave_u & 1) * 256), 4, 0, 0);
-    __builtin_amdgcn_global_load_lds((gptr_t)(a.sw + nn), (lptr_t)(sc + 512 + wave_u * 256), 4, 0, 0);
+    // row scales, column scales, bias (and row map) of this tile, 4 bytes per lane, straight into
+    // LDS; wavefront w fetches 64-entry slice w % (count / 64) of each (duplicates are harmless)
+    const int rs = wave_u % (BM / 64), cs = wave_u % (BN / 64);
+    const int mm = min(m0 + rs * 64 + lane, a.M - 1);
+    const int nn = min(n0 + cs * 64 + lane, a.N - 1);
+    __builtin_amdgcn_global_load_lds((gptr_t)(a.sx + mm), (lptr_t)(sc + C::SX_OFF + rs * 256), 4, 0, 0);
+    __builtin_amdgcn_global_load_lds((gptr_t)(a.sw + nn), (lptr_t)(sc + C::SW_OFF + cs * 256), 4, 0, 0);
     __builtin_amdgcn_global_load_lds((gptr_t)((a.bias ? a.bias : a.sw) + nn),
-                                     (lptr_t)(sc + 1536 + wave_u * 256), 4, 0, 0);
+                                     (lptr_t)(sc + C::BIAS_OFF + cs * 256), 4, 0, 0);
     if (EPI == EPI_RESIDUAL_BF16 && a.dst_row)
-      __builtin_amdgcn_global_load_lds((gptr_t)(a.dst_row + mm),
-                                       (lptr_t)(sc + EP_SCALE_BYTES + (wave_u & 1) * 256), 4, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(a.dst_row + mm), (lptr_t)(sc + C::MAP_OFF + rs * 256), 4, 0, 0);
   }
 
-  i32x16 acc[TM][4];
+  i32x16 acc[TMW][TNW];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TMW; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < TNW; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
   const int frag_chunk = (lh ^ lds_swizzle(lr)) * 16;
-  const int a_off = (wm * 64 + lr) * GLD + frag_chunk;
-  const int b_off = GBM * GLD + (wn * 128 + lr) * GLD + frag_chunk;
+  const int a_off = (wm * (BM / 2) + lr) * GLD + frag_chunk;
+  const int b_off = BM * GLD + (wn * (BN / 2) + lr) * GLD + frag_chunk;
 
   const int nk = a.K / GBK;
   dma_issue(0, 0);
@@ -758,66 +780,79 @@ __global__ __launch_bounds__(256, 3) void gemm_i8_kernel3(GemmArgs a) {
 #pragma unroll
     for (int step = 0; step < 2; ++step) {
       const int flip = step * 32;
-      i32x4 av[TM], bv[4];
+      i32x4 av[TMW], bv[TNW];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (i < TM) av[i] = *reinterpret_cast<const i32x4*>(src + ((a_off + i * 32 * GLD) ^ flip));
-        bv[i] = *reinterpret_cast<const i32x4*>(src + ((b_off + i * 32 * GLD) ^ flip));
-      }
+      for (int i = 0; i < TMW; ++i) av[i] = *reinterpret_cast<const i32x4*>(src + ((a_off + i * 32 * GLD) ^ flip));
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < TNW; ++j) bv[j] = *reinterpret_cast<const i32x4*>(src + ((b_off + j * 32 * GLD) ^ flip));
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+      for (int j = 0; j < TNW; ++j)
+#pragma unroll
+        for (int i = 0; i < TMW; ++i)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], acc[i][j], 0, 0, 0);
     }
   }
 
-  // ---- epilogue, two halves of 64 rows: half h holds MFMA row tile h of both wavefront rows ----
-  // LDS tile row t = wm*32 + rr stands for output row m0 + wm*64 + h*32 + rr
-  const int chunk = tid & 31, rsub = tid >> 5;
+  // ---- epilogue, 64 rows at a time: pass h holds MFMA row tile h of both wavefront rows ----
+  // LDS tile row t = wm*32 + rr stands for output row m0 + wm*(BM/2) + h*32 + rr
+  const int chunk = tid % C::CHUNKS, rsub = tid / C::CHUNKS;
   const int n = n0 + chunk * 8;
   const bool col_ok = n < a.N;  // N % 8 == 0
-  const bool full = m0 + 128 <= a.M && n0 + GBN <= a.N && !(EPI == EPI_RESIDUAL_BF16 && a.dst_row);
+  const bool full = m0 + BM <= a.M && n0 + BN <= a.N && !(EPI == EPI_RESIDUAL_BF16 && a.dst_row);
   unsigned short* outp = reinterpret_cast<unsigned short*>(a.out);
-  const f32x4 swv = *reinterpret_cast<const f32x4*>(sc + 512 + (wn * 128 + 4 * lr) * 4);
-  f32x4 bv4 = {0.f, 0.f, 0.f, 0.f};
+  float swv[TNW], bvv[TNW];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
+  for (int j = 0; j < TNW; ++j) bvv[j] = 0.f;
+#pragma unroll
+  for (int h = 0; h < TMW; ++h) {
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront's LDS reads are done (stores may stay in flight)
-    __builtin_amdgcn_s_barrier();  // operand stages (h = 0) / the first half's tile (h = 1) are no longer read
+    __builtin_amdgcn_s_barrier();  // operand stages (h = 0) / the previous pass's tile are no longer read
     __builtin_amdgcn_sched_barrier(0);
-    if (h == 0 && a.bias) bv4 = *reinterpret_cast<const f32x4*>(sc + 1536 + (wn * 128 + 4 * lr) * 4);
+    if (h == 0) {
+#pragma unroll
+      for (int j = 0; j < TNW; ++j) {
+        swv[j] = *reinterpret_cast<const float*>(sc + C::SW_OFF + (wn * (BN / 2) + TNW * lr + j) * 4);
+        if (a.bias) bvv[j] = *reinterpret_cast<const float*>(sc + C::BIAS_OFF + (wn * (BN / 2) + TNW * lr + j) * 4);
+      }
+    }
     {
-      unsigned char* dst = lds + (wm * 32 + 4 * lh) * EP_STRIDE + (wn * 128 + 4 * lr) * 2;
+      unsigned char* dst = lds + (wm * 32 + 4 * lh) * C::EP_PITCH + (wn * (BN / 2) + TNW * lr) * 2;
       f32x4 sxv[4];
 #pragma unroll
       for (int g = 0; g < 4; ++g)
-        sxv[g] = *reinterpret_cast<const f32x4*>(sc + (wm * 64 + h * 32 + 8 * g + 4 * lh) * 4);
+        sxv[g] = *reinterpret_cast<const f32x4*>(sc + C::SX_OFF + (wm * (BM / 2) + h * 32 + 8 * g + 4 * lh) * 4);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float sxr = sxv[r >> 2][r & 3];
-        float y[4];
+        float y[TNW];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < TNW; ++j) {
           // three separately rounded fp32 operations (no fused multiply-add)
           float t = (float)acc[h][j][r] * sxr;
           t = t * swv[j];
-          y[j] = t + bv4[j];
+          y[j] = t + bvv[j];
         }
-        u32x2 o = {pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3])};
-        if (EPI == EPI_GELU_BF16) {
-          // activation of the bf16-rounded Linear output, as a separate GELU would see it
-          o[0] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[0])), gelu_erf(bf16_hi_to_f32(o[0])));
-          o[1] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[1])), gelu_erf(bf16_hi_to_f32(o[1])));
+        unsigned int o[TNW / 2];
+#pragma unroll
+        for (int j = 0; j < TNW / 2; ++j) {
+          o[j] = pack_bf16x2(y[2 * j], y[2 * j + 1]);
+          if (EPI == EPI_GELU_BF16)  // activation of the bf16-rounded Linear output, as a separate GELU would see it
+            o[j] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[j])), gelu_erf(bf16_hi_to_f32(o[j])));
         }
-        *reinterpret_cast<u32x2*>(dst + (8 * (r >> 2) + (r & 3)) * EP_STRIDE) = o;
+        unsigned char* d = dst + (8 * (r >> 2) + (r & 3)) * C::EP_PITCH;
+        if (TNW == 4) {
+          const u32x2 o2 = {o[0], o[TNW / 2 - 1]};
+          *reinterpret_cast<u32x2*>(d) = o2;
+        } else {
+          *reinterpret_cast<unsigned int*>(d) = o[0];
+        }
       }
     }
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the tile writes have landed
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    // the workgroup walks the 64-row tile 8 rows at a time, 16 bytes per lane
-    const unsigned char* tile = lds + rsub * EP_STRIDE + chunk * 16;
+    // the workgroup walks the 64-row tile ROWS_PER_PASS rows at a time, 16 bytes per lane
+    const unsigned char* tile = lds + rsub * C::EP_PITCH + chunk * 16;
     auto add_residual = [&](u32x4& val, const u32x4& r) {
 #pragma unroll
       for (int c = 0; c < 4; ++c)
@@ -825,36 +860,39 @@ __global__ __launch_bounds__(256, 3) void gemm_i8_kernel3(GemmArgs a) {
         val[c] = pack_bf16x2(bf16_lo_to_f32(val[c]) + bf16_lo_to_f32(r[c]),
                              bf16_hi_to_f32(val[c]) + bf16_hi_to_f32(r[c]));
     };
-    // pass p: tile row t = 8p + rsub -> output row m0 + (t / 32) * 64 + h * 32 + t % 32
+    // pass p: tile row t = ROWS_PER_PASS * p + rsub -> row (t / 32) * (BM / 2) + h * 32 + t % 32 of the tile
+    auto tile_row = [&](int p) {
+      const int t = C::ROWS_PER_PASS * p + rsub;
+      return (t >> 5) * (BM / 2) + h * 32 + (t & 31);
+    };
     if (full) {
-      const int rbase = m0 + h * 32 + rsub;  // + (p / 4) * 64 + (p % 4) * 8
-      u32x4 res[8], val[8];
+      u32x4 res[C::PASSES], val[C::PASSES];
       if (EPI == EPI_RESIDUAL_BF16) {
 #pragma unroll
-        for (int p = 0; p < 8; ++p)
-          res[p] = *reinterpret_cast<const u32x4*>(a.residual + (int64_t)(rbase + (p >> 2) * 64 + (p & 3) * 8) * a.ld_res + n);
+        for (int p = 0; p < C::PASSES; ++p)
+          res[p] = *reinterpret_cast<const u32x4*>(a.residual + (int64_t)(m0 + tile_row(p)) * a.ld_res + n);
       }
 #pragma unroll
-      for (int p = 0; p < 8; ++p) val[p] = *reinterpret_cast<const u32x4*>(tile + 8 * p * EP_STRIDE);
+      for (int p = 0; p < C::PASSES; ++p)
+        val[p] = *reinterpret_cast<const u32x4*>(tile + C::ROWS_PER_PASS * p * C::EP_PITCH);
 #pragma unroll
-      for (int p = 0; p < 8; ++p) {
+      for (int p = 0; p < C::PASSES; ++p) {
         if (EPI == EPI_RESIDUAL_BF16) add_residual(val[p], res[p]);
-        u32x4* op = reinterpret_cast<u32x4*>(outp + (int64_t)(rbase + (p >> 2) * 64 + (p & 3) * 8) * a.ldo + n);
+        u32x4* op = reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + tile_row(p)) * a.ldo + n);
         // an output larger than the last-level cache that is read once (qkv, lin1) is streamed out
         if (a.stream_out) __builtin_nontemporal_store(val[p], op);
         else *op = val[p];
       }
     } else {
 #pragma unroll
-      for (int p = 0; p < 8; ++p) {
-        const int t = 8 * p + rsub;
-        const int row = (t >> 5) * 64 + h * 32 + (t & 31);  // row inside the 128-row tile
+      for (int p = 0; p < C::PASSES; ++p) {
+        const int row = tile_row(p);
         int dr = -1;
         if (m0 + row < a.M && col_ok) {
           dr = m0 + row;
-          if (EPI == EPI_RESIDUAL_BF16 && a.dst_row) dr = *reinterpret_cast<const int*>(sc + EP_SCALE_BYTES + row * 4);
+          if (EPI == EPI_RESIDUAL_BF16 && a.dst_row) dr = *reinterpret_cast<const int*>(sc + C::MAP_OFF + row * 4);
         }
-        u32x4 val = *reinterpret_cast<const u32x4*>(tile + 8 * p * EP_STRIDE);
+        u32x4 val = *reinterpret_cast<const u32x4*>(tile + C::ROWS_PER_PASS * p * C::EP_PITCH);
         if (dr >= 0) {
           if (EPI == EPI_RESIDUAL_BF16)
             add_residual(val, *reinterpret_cast<const u32x4*>(a.residual + (int64_t)dr * a.ld_res + n));
@@ -957,17 +995,28 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   // the three-workgroups-per-CU form of the main kernel (SAMFAST_GEMM_WG3=0: two per CU)
   const char* wg3 = getenv("SAMFAST_GEMM_WG3");
   if (!tail && !generic && tm == 2 && epi != EPI_I32 && !(wg3 && atoi(wg3) == 0)) {
-    switch (epi) {
-      case EPI_SCALE_BIAS_BF16:
-        hipLaunchKernelGGL((gemm_i8_kernel3<EPI_SCALE_BIAS_BF16>), dim3(grid), dim3(256), 0, stream, a);
-        break;
-      case EPI_GELU_BF16:
-        hipLaunchKernelGGL((gemm_i8_kernel3<EPI_GELU_BF16>), dim3(grid), dim3(256), 0, stream, a);
-        break;
-      default:
-        hipLaunchKernelGGL((gemm_i8_kernel3<EPI_RESIDUAL_BF16>), dim3(grid), dim3(256), 0, stream, a);
-        break;
+    // 64 x 128 tiles when 128 x 256 ones would leave more than half of the 768 workgroup slots of
+    // the GPU empty (SAMFAST_GEMM_TILE=64 / 128 forces either)
+    const char* ft = getenv("SAMFAST_GEMM_TILE");
+    const bool small = ft ? atoi(ft) == 64 : total < 384;
+    if (small) {
+      a.tiles_m = (int)((M + 63) / 64);
+      a.tiles_n = (N + 127) / 128;
+      a.group_m = a.tiles_n <= 6 ? 1 : 1024 / 64;
     }
+    const int64_t total3 = (int64_t)a.tiles_m * a.tiles_n;
+    const unsigned int grid3 = (unsigned int)(((total3 + 7) / 8) * 8);
+#define SF_GEMM3(E)                                                                                          \
+  do {                                                                                                       \
+    if (small) hipLaunchKernelGGL((gemm_i8_kernel3<E, 64, 128>), dim3(grid3), dim3(256), 0, stream, a);      \
+    else hipLaunchKernelGGL((gemm_i8_kernel3<E, 128, 256>), dim3(grid3), dim3(256), 0, stream, a);           \
+  } while (0)
+    switch (epi) {
+      case EPI_SCALE_BIAS_BF16: SF_GEMM3(EPI_SCALE_BIAS_BF16); break;
+      case EPI_GELU_BF16: SF_GEMM3(EPI_GELU_BF16); break;
+      default: SF_GEMM3(EPI_RESIDUAL_BF16); break;
+    }
+#undef SF_GEMM3
     return check_launch("gemm_i8_kernel3");
   }
   if (tail) {

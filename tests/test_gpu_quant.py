@@ -482,9 +482,11 @@ def test_gemm_with_output_quantiser_in_place_residual():
 @pytest.mark.parametrize("M,N,K,epi", [(300, 1280, 1280, "residual"), (1000, 3840, 1280, "none"),
                                        (513, 5120, 1280, "gelu"), (260, 1280, 5120, "residual_scatter")])
 def test_gemm_two_and_three_workgroups_per_cu_agree(monkeypatch, M, N, K, epi):
-    """The main GEMM kernel exists in two forms - three workgroups per CU (single-buffered fragments,
-    two LDS stages, epilogue staged in two halves; the default) and two per CU (SAMFAST_GEMM_WG3=0) -
-    that must agree bit for bit with each other (and, by the other tests, with the oracle)."""
+    """The main GEMM kernel exists in three forms - three workgroups per CU with 128 x 256 tiles
+    (single-buffered fragments, two LDS stages, epilogue staged 64 rows at a time; the default), the
+    same with 64 x 128 tiles (small launches, SAMFAST_GEMM_TILE=64) and two per CU
+    (SAMFAST_GEMM_WG3=0) - that must agree bit for bit with each other (and, by the other tests,
+    with the oracle)."""
     from samfast_amd import _lib, ops
     g = torch.Generator().manual_seed(M + N)
     x = torch.randn((M, K), generator=g).to(torch.bfloat16).cuda()
@@ -503,9 +505,12 @@ def test_gemm_two_and_three_workgroups_per_cu_agree(monkeypatch, M, N, K, epi):
             perm[5] = -1
             kw["dst_row"] = perm.cuda()
     outs = []
-    for wg3 in ("1", "0"):
+    # three per CU with 128 x 256 tiles, three (or more) per CU with 64 x 128 tiles, two per CU
+    for wg3, tile in (("1", "128"), ("1", "64"), ("0", "128")):
         monkeypatch.setenv("SAMFAST_GEMM_WG3", wg3)
+        monkeypatch.setenv("SAMFAST_GEMM_TILE", tile)
         out = torch.zeros_like(kw["residual"]) if "residual" in kw else None
         outs.append(ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L, out=out, **kw).clone())
     torch.cuda.synchronize()
-    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
+    assert torch.equal(outs[1].view(torch.int16), outs[2].view(torch.int16))
