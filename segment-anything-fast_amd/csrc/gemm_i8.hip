@@ -998,7 +998,8 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
     // 64 x 128 tiles when 128 x 256 ones would leave more than half of the 768 workgroup slots of
     // the GPU empty (SAMFAST_GEMM_TILE=64 / 128 forces either)
     const char* ft = getenv("SAMFAST_GEMM_TILE");
-    const bool small = ft ? atoi(ft) == 64 : total < 384;
+    const char* fb = getenv("SAMFAST_GEMM_SMALL_BELOW");  // tuning aid: the tile-count threshold
+    const bool small = ft ? atoi(ft) == 64 : total < (fb ? atoi(fb) : 384);
     if (small) {
       a.tiles_m = (int)((M + 63) / 64);
       a.tiles_n = (N + 127) / 128;
