@@ -514,3 +514,51 @@ def test_gemm_two_and_three_workgroups_per_cu_agree(monkeypatch, M, N, K, epi):
     torch.cuda.synchronize()
     assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
     assert torch.equal(outs[1].view(torch.int16), outs[2].view(torch.int16))
+
+
+def test_gelu_epilogue_all_bf16_inputs(monkeypatch):
+    """Every bf16 bit pattern through the GELU epilogue.  Zero weights and bias[n] = the bf16
+    value with bits n make column n of the Linear output that value, so one launch evaluates the
+    activation on all 65 536 inputs.  The three forms of the kernel (128 x 256 and 64 x 128 tiles
+    at three workgroups per CU, two workgroups per CU) must give the same bits, for even and odd
+    counts of k tiles, and inside |x| <= 6 every result is within one bf16 step of the erf GELU."""
+    from samfast_amd import _lib, ops
+    N = 65536
+    pat = torch.arange(N, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)  # bits n
+    bias = pat.float().cuda()
+    outs = {}
+    for K in (256, 320):
+        M = 128
+        xq = torch.ones((M, K), dtype=torch.int8).cuda()
+        sx = torch.ones((M,), dtype=torch.float32).cuda()
+        wq = torch.zeros((N, K), dtype=torch.int8).cuda()
+        sw = torch.ones((N,), dtype=torch.float32).cuda()
+        for name, wg3, tile in (("large", "1", "128"), ("small", "1", "64"), ("two", "0", "128")):
+            monkeypatch.setenv("SAMFAST_GEMM_WG3", wg3)
+            monkeypatch.setenv("SAMFAST_GEMM_TILE", tile)
+            y = ops.gemm_i8_fused(xq, sx, wq, sw, bias, _lib.EPILOGUE_GELU)
+            torch.cuda.synchronize()
+            assert torch.equal(y[0].view(torch.int16), y[M - 1].view(torch.int16))
+            outs[(K, name)] = y[0].cpu()
+    want = outs[(256, "two")]
+    finite = torch.isfinite(pat.float())
+    for key, got in outs.items():
+        assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), key
+        same = (got.view(torch.int16) == want.view(torch.int16)) | torch.isnan(want.float())
+        assert bool(same.all()), (key, int((~same).sum()))
+    x = pat.float()
+    assert bool(torch.isnan(want.float()[torch.isnan(x)]).all())  # a NaN stays a NaN
+    ref = torch.nn.functional.gelu(x.double()).to(torch.bfloat16)
+    inside = finite & (x.abs() <= 6)
+    g, r = want.float()[inside], ref.float()[inside]
+    step = torch.maximum(r.abs(), torch.tensor(2.0 ** -126)) * 2.0 ** -7  # one bf16 step at r or more
+    assert bool(((g - r).abs() <= step).all())
+    # beyond 6 the kernels hold Phi(-|x|) at Phi(-6) = 1e-9: x itself on the positive side, and on
+    # the negative side -|x| * 1e-9 where the exact value has already fallen below 6e-9
+    big = finite & (x > 6)
+    assert torch.equal(want[big].view(torch.int16), pat[big].view(torch.int16))
+    low = finite & (x < -6)
+    assert bool((want.float()[low] <= 0).all()) and bool((want.float()[low].abs() <= x[low].abs() * 1.1e-9).all())
+    # over the values a Linear output takes in practice 99.5 % are the correctly rounded result
+    usual = finite & (x.abs() >= 2.0 ** -6) & (x.abs() <= 6)
+    assert (want.float()[usual] == ref.float()[usual]).float().mean() >= 0.995
