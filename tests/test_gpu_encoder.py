@@ -93,6 +93,32 @@ def test_vit_h_slice_vs_pytorch_rocm_bf16():
     assert c >= COSINE_MIN
 
 
+def test_vit_l_slice_vs_oracle():
+    """ViT-L shapes (embed 1024, 16 heads of 64 channels, MLP 4096), 3 blocks with the last one
+    global, bs 2: attention kernels + int8 linears (fused block) against the oracle that
+    quantises the same way on the CPU.  Bar: cosine >= 0.999 per image."""
+    from samfast_amd import apply_dynamic_quant
+    from samfast_amd.modeling import ImageEncoderViT
+    from samfast_amd.synthetic import init_encoder_weights, make_images
+    enc = ImageEncoderViT(depth=3, embed_dim=1024, num_heads=16, global_attn_indexes=(2,),
+                          window_size=14, use_rel_pos=True, mlp_ratio=4,
+                          norm_layer=partial(torch.nn.LayerNorm, eps=1e-6))
+    sd = {k: v.clone() for k, v in init_encoder_weights(enc, seed=5).items()}
+    x = make_images(2, seed=6).to(torch.bfloat16)
+    cfg = oe.EncoderConfig(1024, 3, 16, (2,))
+    lin = lambda a, w, b: oq.dynamic_int8_linear(a, w, b).float()
+    with torch.no_grad():
+        ref = oe.encoder_forward(_rounded(sd), x.float(), cfg, linear=lin, use_sdpa=True)
+        enc = enc.eval().to(torch.bfloat16).cuda()
+        apply_dynamic_quant(enc)
+        assert all(b._int8_fused_ok(torch.empty(2, 64, 64, 1024, dtype=torch.bfloat16, device="cuda"))
+                   for b in enc.blocks)
+        out = enc(x.cuda())
+    c = _cos(out, ref)
+    print(f"vit_l slice int8: cosine vs quantised oracle {c:.6f}", flush=True)
+    assert torch.isfinite(out.float()).all() and c >= COSINE_MIN
+
+
 def test_predictor_set_torch_image():
     import samfast_amd
     from samfast_amd.synthetic import init_encoder_weights
