@@ -85,10 +85,29 @@ class ImageEncoderViT(nn.Module):
             LayerNorm2d(out_chans),
         )
 
+    # images per pass through the blocks; None = as many as the int8 kernels can address
+    max_images_per_pass: Optional[int] = None
+
+    def images_per_pass(self, x: torch.Tensor) -> int:
+        """The int8 GEMMs and the row quantiser address an activation of M rows and K columns with
+        32-bit offsets (M * K < 2^31).  The widest one is lin2's input, 4C per token: 102 images of
+        64 x 64 tokens at ViT-H.  Images are independent, so a larger batch goes through the blocks
+        in passes of at most that many."""
+        if self.max_images_per_pass is not None:
+            return max(1, int(self.max_images_per_pass))
+        from ..quant import Int8LinearBase
+        widest = max((m.in_features for m in self.modules() if isinstance(m, Int8LinearBase)), default=0)
+        if widest == 0:
+            return x.shape[0]
+        return max(1, (2 ** 31 - 1) // (x.shape[1] * x.shape[2] * widest))
+
     def forward_blocks(self, x: torch.Tensor) -> torch.Tensor:
         """The transformer blocks on (B, H, W, C) tokens.  Consecutive blocks on the fused int8
         path are chained: a block's lin2 launch also runs the next block's norm1 and the qkv
         Linear's quantiser on the rows it has just written."""
+        per_pass = self.images_per_pass(x)
+        if x.shape[0] > per_pass:
+            return torch.cat([self.forward_blocks(x[i:i + per_pass]) for i in range(0, x.shape[0], per_pass)])
         carry = None
         for i, blk in enumerate(self.blocks):
             if not blk._int8_fused_ok(x):

@@ -313,6 +313,29 @@ def test_vit_h_batch_16_blocks_bitwise_equal_batch_2_runs():
     assert out.shape == (16, 256, 64, 64) and torch.isfinite(out.float()).all()
 
 
+def test_oversized_batch_goes_through_the_blocks_in_passes():
+    """The int8 kernels address an activation with 32-bit offsets, which caps a pass through the
+    blocks at 102 images for ViT-H; a larger batch is cut into passes.  Forced here with a cap of
+    2 on 5 images of a two-block ViT-B-shaped encoder: same bits as one pass."""
+    from samfast_amd import apply_dynamic_quant
+    from samfast_amd.modeling import ImageEncoderViT
+    from samfast_amd.synthetic import init_encoder_weights, make_images
+    enc = ImageEncoderViT(depth=2, embed_dim=768, num_heads=12, global_attn_indexes=(1,),
+                          window_size=14, use_rel_pos=True, mlp_ratio=4,
+                          norm_layer=partial(torch.nn.LayerNorm, eps=1e-6))
+    init_encoder_weights(enc, seed=7)
+    enc = enc.eval().to(torch.bfloat16).cuda()
+    apply_dynamic_quant(enc)
+    with torch.no_grad():
+        x0 = _trunk_input(enc, make_images(5, seed=8).to(torch.bfloat16).cuda())
+        assert enc.images_per_pass(x0) == (2 ** 31 - 1) // (4096 * 3072)
+        whole = enc.forward_blocks(x0.clone())
+        enc.max_images_per_pass = 2
+        parts = enc.forward_blocks(x0.clone())
+    assert parts.shape == whole.shape
+    assert torch.equal(parts.view(torch.int16), whole.view(torch.int16))
+
+
 def test_vit_h_batch_32_sparse_mlp_bitwise_equals_dense_kernels_on_pruned_weights():
     """The int8 + 2:4 configuration at its real batch (32 images, all 32 blocks): the sparse matrix
     cores on the packed lin1 / lin2 weights must reproduce, bit for bit, the dense int8 kernels run on
