@@ -538,7 +538,12 @@ struct WindowCfg {
   static constexpr bool ONES_ROW = HD % 32 != 0;
   static constexpr int XSTR = 50;              // bf16 elements per scratch row: 32 products stored in reverse + read-ahead room; 25 words: odd, no bank conflicts
   static constexpr int XBYTES_WAVE = 32 * XSTR * 2;  // gather scratch, aliases the V area before V arrives
-  static constexpr int LDS_BYTES = KBYTES + VBYTES;
+  // the 0/1 indicator operands of the bias MFMAs as a table behind V: entry e < 16 is the one-hot
+  // vector of slot e (16 elements of 2 bytes), entry 16 all zeros; a lane reads its half by one
+  // 16-byte LDS read instead of building it from compares
+  static constexpr int HOT_ENTRIES = 17;
+  static constexpr int HOT_BYTES = HOT_ENTRIES * 32;
+  static constexpr int LDS_BYTES = KBYTES + VBYTES + HOT_BYTES;
   static_assert(WAVES * XBYTES_WAVE <= VBYTES, "gather scratch must fit in the V area");
   static_assert(NT <= WAVES, "one query tile per wavefront");
 };
@@ -563,11 +568,14 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
   __shared__ __attribute__((aligned(16))) unsigned char lds[C::LDS_BYTES];
   unsigned char* kl = lds;
   unsigned char* vl = lds + C::KBYTES;
+  unsigned char* hot = lds + C::KBYTES + C::VBYTES;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 31, lh = lane >> 5;
   const int N = a.N;
+  // the indicator table (read only after the barrier that follows the arrival of K)
+  if (tid < 2 * C::HOT_ENTRIES) *reinterpret_cast<u32x4*>(hot + tid * 16) = onehot_x8<T>(tid >> 1, tid & 1);
   // all heads of a window run on one XCD: their 2*HD-byte slices of a token share cache lines
   const unsigned int total = (unsigned int)((a.ws > 0 ? a.B * a.wins_x * a.wins_y : a.B) * a.nH);
   const int bh = (int)xcd_contiguous_id(blockIdx.x, total);
@@ -806,8 +814,9 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
           acc = T::mfma(av, qf[ks], acc);
         }
         const int nh = div_gw(min(n, 255));
-        const u32x4 ih = onehot_x8<T>(n < N ? nh : 15, lh);
-        const u32x4 iw = onehot_x8<T>(n < N ? n - nh * a.gw : 99, lh);
+        // slot 15 of the row part is the padding mask; a padding key has no column
+        const u32x4 ih = *reinterpret_cast<const u32x4*>(hot + (n < N ? nh : 15) * 32 + lh * 16);
+        const u32x4 iw = *reinterpret_cast<const u32x4*>(hot + (n < N ? n - nh * a.gw : 16) * 32 + lh * 16);
         acc = T::mfma(ih, bh_op, acc);
         acc = T::mfma(iw, bw_op, acc);
 
