@@ -592,12 +592,14 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
   }
   // token n of the window -> row index inside the (b, head) slice, or -1 for a padding token
   // n / gw for 0 <= n < 256 and gw <= 16 by multiplication (exact in that range)
+  // (24-bit multiplies: full-rate instructions, and every product here is below 2^24)
   const int gw_magic = 65536 / a.gw + 1;
-  auto div_gw = [&](int n) { return (n * gw_magic) >> 16; };
+  auto div_gw = [&](int n) { return (int)(__umul24((unsigned int)n, (unsigned int)gw_magic) >> 16); };
+  auto times_gw = [&](int r) { return (int)__umul24((unsigned int)r, (unsigned int)a.gw); };
   auto tok_of = [&](int n) {
     if (a.ws <= 0) return n;
     const int ny = div_gw(n);
-    const int y = win_y0 + ny, x = win_x0 + n - ny * a.gw;
+    const int y = win_y0 + ny, x = win_x0 + n - times_gw(ny);
     return (y < a.img_h && x < a.img_w) ? y * a.img_w + x : -1;
   };
 
@@ -679,7 +681,7 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
   //      slot 8*lh + e.  The gather scratch lives where K will be stored afterwards ----------
   u32x4 bias_hv, bias_wv;
   {
-    const int qh = div_gw(qc), qw = qc - qh * a.gw;
+    const int qh = div_gw(qc), qw = qc - times_gw(qh);
     unsigned int bhw[4] = {0u, 0u, 0u, 0u}, bww[4] = {0u, 0u, 0u, 0u};
     if (FUSED) {
       unsigned short* X = reinterpret_cast<unsigned short*>(vl + wave * C::XBYTES_WAVE);
@@ -804,21 +806,31 @@ __global__ __launch_bounds__(WindowCfg<HD>::THREADS, 2) void attn_window_kernel(
     for (int nt = 0; nt < C::NT; ++nt) {
       if (32 * nt < N) {  // uniform
         const int n = 32 * nt + lr;
-        const int nc = min(n, N - 1);
+        // A key tile that lies inside the window whole (all but the last one: 6 of 7 at 196 keys)
+        // needs neither the clamp of its K rows nor the selects of the padding mask; its K
+        // addresses are then the lane's tile-0 address plus a constant.
+        auto score_tile = [&](auto whole_c) {
+          constexpr bool WHOLE = decltype(whole_c)::value;
+          const int nc = WHOLE ? n : min(n, N - 1);
+          f32x16 sacc;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+#pragma unroll
+          for (int ks = 0; ks < C::KS; ++ks) {
+            const u32x4 av = *reinterpret_cast<const u32x4*>(kl + (nc * C::KSTR + 16 * ks + 8 * lh) * 2);
+            sacc = T::mfma(av, qf[ks], sacc);
+          }
+          const int nh = div_gw(WHOLE ? n : min(n, 255));
+          const bool real = WHOLE || n < N;
+          // slot 15 of the row part is the padding mask; a padding key has no column
+          const u32x4 ih = *reinterpret_cast<const u32x4*>(hot + (real ? nh : 15) * 32 + lh * 16);
+          const u32x4 iw = *reinterpret_cast<const u32x4*>(hot + (real ? n - times_gw(nh) : 16) * 32 + lh * 16);
+          sacc = T::mfma(ih, bh_op, sacc);
+          return T::mfma(iw, bw_op, sacc);
+        };
         f32x16 acc;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < C::KS; ++ks) {
-          const u32x4 av = *reinterpret_cast<const u32x4*>(kl + (nc * C::KSTR + 16 * ks + 8 * lh) * 2);
-          acc = T::mfma(av, qf[ks], acc);
-        }
-        const int nh = div_gw(min(n, 255));
-        // slot 15 of the row part is the padding mask; a padding key has no column
-        const u32x4 ih = *reinterpret_cast<const u32x4*>(hot + (n < N ? nh : 15) * 32 + lh * 16);
-        const u32x4 iw = *reinterpret_cast<const u32x4*>(hot + (n < N ? n - nh * a.gw : 16) * 32 + lh * 16);
-        acc = T::mfma(ih, bh_op, acc);
-        acc = T::mfma(iw, bw_op, acc);
+        if (32 * nt + 32 <= N) acc = score_tile(std::true_type{});  // uniform
+        else acc = score_tile(std::false_type{});
 
         float mx = acc[0];
 #pragma unroll
