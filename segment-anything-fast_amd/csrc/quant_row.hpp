@@ -61,9 +61,14 @@ SF_DEVICE float wave_max_nonneg(float v) {
 }
 
 // EPC (4 or 8) values -> EPC int8 codes packed in EPC bytes.
-// Rounding: adding 1.5 * 2^23 to r (|r| <= 127) leaves rint(r) - half to even - in the low
-// mantissa bits, so the low byte of the sum's bit pattern is the int8 code; subtracting the
-// constant again gives rint(r) as a float for the near-tie test.
+// The code wanted is rint(fl(v / scale)) with the correctly rounded IEEE quotient.  The cheap
+// route works on p = v * inv_scale (inv_scale = fl(1 / scale)), taken exactly inside fused
+// multiply-adds: m = fl(p + 1.5 * 2^23) holds rint(p) - half to even - in its low mantissa bits
+// (|p| <= 127 (1 + 2^-23)), so the low byte of m's bit pattern is the int8 code of p, and
+// d = fl(p - (m - 1.5 * 2^23)) is p - rint(p) to 3e-8.  p differs from v / scale by at most
+// 127 * 2^-24 (the rounding of inv_scale) and fl(v / scale) from v / scale by as much: 1.6e-5
+// together.  Unless p lies within that distance of a half-integer, rint(p) is the wanted code;
+// chunks with a |d| above 0.5 - 2.5e-5 are redone with the true division.
 // Returns true when the chunk holds a NaN: the comparison that finds near-ties is written so
 // that a NaN product also takes the slow path, where the chunk's values are looked at once more;
 // the common path pays nothing for it.
@@ -74,10 +79,9 @@ SF_DEVICE bool quantize_chunk(const float (&v)[EPC], float scale, float inv_scal
   bool near_tie = false, saw_nan = false;
 #pragma unroll
   for (int e = 0; e < EPC; ++e) {
-    const float r = v[e] * inv_scale;
-    m[e] = r + kMagic;
-    const float d = r - (m[e] - kMagic);  // r - rint(r), exact
-    near_tie |= !(fabsf(d) <= 0.5f - 1e-4f);  // also true for a NaN
+    m[e] = fmaf(v[e], inv_scale, kMagic);
+    const float d = fmaf(v[e], inv_scale, kMagic - m[e]);  // kMagic - m[e] = -rint(p), exact
+    near_tie |= !(fabsf(d) <= 0.5f - 2.5e-5f);  // also true for a NaN
   }
   if (near_tie) {
 #pragma unroll
