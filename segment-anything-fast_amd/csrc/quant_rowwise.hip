@@ -10,10 +10,10 @@
 // Algorithmic traffic: 2 bytes read + 1 byte written per element + 4 bytes of scale.
 //
 // q = rint(x / s) must equal the IEEE division bit for bit.  Most elements take a
-// cheap route: r = x * (1/s) differs from x / s by a few ulp, so rint(r) can only
-// differ when r lies within 1e-4 of a half-integer; only those elements (and their
-// 8-element chunk) are redone with the true division.  |x| <= absmax makes
-// |x / s| <= 127 by construction, so no clamp is needed.
+// cheap route: the exact product x * fl(1/s) differs from fl(x / s) by at most 1.6e-5, so
+// its rint can only differ when it lies within that distance of a half-integer; only those
+// elements (and their 8-element chunk) are redone with the true division (quant_row.hpp).
+// |x| <= absmax makes |x / s| <= 127 by construction, so no clamp is needed.
 #include "quant_row.hpp"
 
 namespace samfast {
