@@ -249,6 +249,43 @@ def mfma_ceiling():
         gemm[name] = round(2.0 * M * N * K * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e15, 3)
         del xq, wq
     res["gemm_i8_kernel_same_shape_different_data"] = gemm
+
+    # how much vector work fits under another wavefront's MFMAs on the same SIMD: one 8-wavefront
+    # workgroup per CU, wavefronts 0-3 only MFMAs, wavefronts 4-7 only vector instructions, sized so
+    # that either side alone takes the same time; overlap = (alone_a + alone_b - both) / min(alone)
+    def timed(kind, mfma_rounds, vector_rounds):
+        launch = lambda: _lib.check(lib.samfast_bench_mfma_valu_overlap(
+            kind, buf.data_ptr(), 256, mfma_rounds, vector_rounds, out.data_ptr(), stream), "bench_mfma_valu_overlap")
+        launch()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            launch()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1))
+        return best
+
+    overlap = {"what": "256 workgroups of 8 wavefronts: wavefronts 0-3 v_mfma_f32_32x32x16_bf16 only, wavefronts 4-7 "
+                       "(their SIMD partners) vector instructions only; ms alone, ms together, share of the shorter "
+                       "side that ran under the other"}
+    rounds = 20000
+    # on all-zero MFMA operands the matrix pipe draws little power, so the clock does not fall when
+    # the vector side joins: that pair isolates the issue limit from the power limit
+    for data in ("zeros", "random_normal"):
+        buf = operands[1][data]
+        t_mfma = timed(0, rounds, 0)
+        for kind, name in ((0, "v_fma_f32"), (1, "v_exp_f32_then_v_mul_f32")):
+            probe = timed(kind, 0, 2000)
+            vr = max(1, int(2000 * t_mfma / probe))
+            t_vec = timed(kind, 0, vr)
+            t_both = timed(kind, rounds, vr)
+            overlap[f"{name}_mfma_operands_{data}"] = {
+                "mfma_alone_ms": round(t_mfma, 3), "vector_alone_ms": round(t_vec, 3), "together_ms": round(t_both, 3),
+                "overlap": round((t_mfma + t_vec - t_both) / min(t_mfma, t_vec), 3)}
+    res["mfma_and_vector_wavefronts_on_one_simd"] = overlap
     return res
 
 

@@ -304,6 +304,19 @@ int samfast_bench_mfma_ceiling(
     int instruction, const void* operands, int workgroups, int iters,
     int64_t* host_ops_out, void* scratch_out, void* stream);
 
+/*
+ * Measurement aid, no counterpart in the reference: how much vector work runs in the shadow of
+ * another wavefront's matrix instructions on the same SIMD.  Workgroups of 512 threads, one per
+ * CU: wavefronts 0-3 run `mfma_rounds` rounds of eight independent v_mfma_f32_32x32x16_bf16 on
+ * operands held in registers, wavefronts 4-7 (their SIMD partners) `vector_rounds` rounds of 64
+ * independent vector instructions - vector_kind 0: v_fma_f32, 1: v_exp_f32 + v_mul_f32.  Either
+ * count may be 0, which times one side alone.  `operands`: at least 8 KiB (two 16-byte vectors for
+ * each of 256 lanes); `scratch_out`: 2 KiB the kernel may write.  bench.py --mfma-ceiling uses it.
+ */
+int samfast_bench_mfma_valu_overlap(
+    int vector_kind, const void* operands, int workgroups, int mfma_rounds, int vector_rounds,
+    void* scratch_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

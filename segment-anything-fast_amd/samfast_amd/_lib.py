@@ -48,6 +48,7 @@ _SIGNATURES = {
         _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _i32,
                _ptr, _i64, _i32, _ptr]),
     "samfast_bench_mfma_ceiling": (_i32, [_i32, _ptr, _i32, _i32, ctypes.POINTER(_i64), _ptr, _ptr]),
+    "samfast_bench_mfma_valu_overlap": (_i32, [_i32, _ptr, _i32, _i32, _i32, _ptr, _ptr]),
 }
 
 EPILOGUE_NONE, EPILOGUE_GELU, EPILOGUE_RESIDUAL = 0, 1, 2

@@ -562,3 +562,25 @@ def test_gelu_epilogue_all_bf16_inputs(monkeypatch):
     # over the values a Linear output takes in practice 99.5 % are the correctly rounded result
     usual = finite & (x.abs() >= 2.0 ** -6) & (x.abs() <= 6)
     assert (want.float()[usual] == ref.float()[usual]).float().mean() >= 0.995
+
+
+def test_measurement_aids_run_and_check_their_arguments():
+    """The two bench-only entry points (MFMA-only loops; MFMA and vector wavefronts sharing SIMDs)
+    launch, finish and reject bad arguments; what they measure is read by bench.py --mfma-ceiling."""
+    import ctypes
+    from samfast_amd import _lib
+    lib = _lib.load()
+    buf = torch.randn(8 * 256 * 8, device="cuda").to(torch.bfloat16)
+    out = torch.zeros(1024, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    ops_done = ctypes.c_int64(0)
+    for instr in (0, 1):
+        assert lib.samfast_bench_mfma_ceiling(instr, buf.data_ptr(), 8, 10, ctypes.byref(ops_done), out.data_ptr(), stream) == 0
+        assert ops_done.value == 8 * 4 * 10 * 8 * 2 * 32 * 32 * (32 if instr == 0 else 16)
+    for kind, mr, vr in ((0, 10, 10), (1, 10, 10), (0, 0, 10), (1, 10, 0), (0, 0, 0)):
+        assert lib.samfast_bench_mfma_valu_overlap(kind, buf.data_ptr(), 8, mr, vr, out.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    assert int(out.abs().sum()) == 0  # the kernels write nothing
+    assert lib.samfast_bench_mfma_valu_overlap(2, buf.data_ptr(), 8, 1, 1, out.data_ptr(), stream) == -1  # SAMFAST_E_INVALID
+    assert lib.samfast_bench_mfma_valu_overlap(0, None, 8, 1, 1, out.data_ptr(), stream) == -1  # SAMFAST_E_INVALID
+    assert lib.samfast_bench_mfma_valu_overlap(0, buf.data_ptr(), 8, -1, 1, out.data_ptr(), stream) == -1  # SAMFAST_E_INVALID
