@@ -61,6 +61,9 @@ def parse():
     p.add_argument("--no-mfma-ceiling", action="store_true", help="skip the matrix-instruction-only loops")
     p.add_argument("--mfma-ceiling", action="store_true",
                    help="run ONLY the matrix-instruction-only loops and print their JSON object")
+    p.add_argument("--gemm-variants", action="store_true",
+                   help="run ONLY the int8 GEMM variant table: the four ViT-H linears at 65536 rows under every "
+                        "kernel-variant knob, on all-zero and on model-like codes, and print its JSON object")
     p.add_argument("--bf16-linears", action="store_true", help="keep nn.Linear (attention kernels only)")
     p.add_argument("--sparse-mlp", action="store_true",
                    help="lin1 / lin2 magnitude-pruned 2:4 on the sparse int8 matrix cores (the int8 + 2:4 "
@@ -289,6 +292,58 @@ def mfma_ceiling():
     return res
 
 
+def gemm_variants(batch=16, width=1280):
+    """The four Linears of a ViT-H block at batch * 4096 rows (K-block major operands, the epilogue the
+    encoder uses) under each variant of the int8 GEMM kernel, ten launches back to back after three
+    warm-up launches, events on the launch stream; on all-zero codes (no operand toggling: the clock
+    stays up, what is left is the kernel's structure) and on Gaussian codes like the encoder's."""
+    import torch
+    from samfast_amd import _lib, ops
+    dev = torch.device("cuda:0")
+    M = batch * 4096
+    g = torch.Generator(device="cuda").manual_seed(11)
+    variants = [("three_workgroups_per_cu (default)", {}),
+                ("two_workgroups_per_cu", {"SAMFAST_GEMM_WG3": 0}),
+                ("persistent (where built, else the default)", {"SAMFAST_GEMM_PERSIST": 1})]
+    shapes = [("qkv", 3 * width, width, _lib.EPILOGUE_NONE), ("proj", width, width, _lib.EPILOGUE_RESIDUAL),
+              ("lin1", 4 * width, width, _lib.EPILOGUE_GELU), ("lin2", width, 4 * width, _lib.EPILOGUE_RESIDUAL)]
+    res = {"what": f"gemm_i8 at M={M}, us per launch (10 back to back) and TOP/s, per variant knob, on "
+                   "all-zero / Gaussian int8 codes", "rows": {}}
+    for name, N, K, epi in shapes:
+        sx = torch.full((M,), 0.01, device=dev)
+        sw = torch.full((N,), 0.001, device=dev)
+        bias = torch.zeros((N,), device=dev)
+        y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        resid = torch.randn((M, N), device=dev, generator=g).to(torch.bfloat16) if epi == _lib.EPILOGUE_RESIDUAL else None
+        row = {}
+        for data in ("zeros", "gaussian"):
+            if data == "zeros":
+                xq = torch.zeros((K // 64, M, 64), dtype=torch.int8, device=dev)
+                wq = torch.zeros((K // 64, N, 64), dtype=torch.int8, device=dev)
+            else:
+                xq = (torch.randn((K // 64, M, 64), device=dev, generator=g) * 28).round().clamp(-127, 127).to(torch.int8)
+                wq = (torch.randn((K // 64, N, 64), device=dev, generator=g) * 28).round().clamp(-127, 127).to(torch.int8)
+            run = lambda: ops.gemm_i8_fused(xq, sx, wq, sw, bias, epi, residual=resid, out=y, layout=_lib.LAYOUT_KB64)
+            for label, knobs in variants:
+                with _lib.knobs(**knobs):
+                    for _ in range(3):
+                        run()
+                    torch.cuda.synchronize()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(10):
+                        run()
+                    e1.record()
+                    torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 100.0
+                row.setdefault(label, {})[data] = {"us": round(us, 1), "TOP/s": round(2.0 * M * N * K / us / 1e6, 1)}
+            del xq, wq
+        res["rows"][f"{name} {M}x{N}x{K}"] = row
+        del y, resid
+    torch.cuda.empty_cache()
+    return res
+
+
 def run_config(model, batch, steps, warmup, sparse_mlp=False, bf16_linears=False, graph=False,
                gpu_baseline=True, calibration_copy=False, yardsticks=False, also_graph=False,
                compiled_baseline=False):
@@ -464,6 +519,9 @@ def main():
 
     if args.mfma_ceiling:
         print(json.dumps({"mfma_ceiling": mfma_ceiling()}))
+        return
+    if args.gemm_variants:
+        print(json.dumps({"gemm_variants": gemm_variants()}))
         return
 
     main_run, sd_fp32 = run_config(

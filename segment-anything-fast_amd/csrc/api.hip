@@ -1,8 +1,12 @@
 // Library-level entry points: version, architecture, per-thread error text.
+#include <pthread.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
 
 #include "samfast_internal.hpp"
+#include "samfast_bench.h"
 
 namespace samfast {
 
@@ -24,7 +28,37 @@ int check_launch(const char* what) {
   return SAMFAST_OK;
 }
 
+static const char* const kKnobNames[KNOB_COUNT] = {
+    "SAMFAST_GEMM_TM",      "SAMFAST_GEMM_WG3",    "SAMFAST_GEMM_TILE", "SAMFAST_GEMM_SMALL_BELOW",
+    "SAMFAST_GEMM_PERSIST", "SAMFAST_GEMM_SPLITK", "SAMFAST_ATTN_WAVES"};
+static int g_knobs[KNOB_COUNT];
+static pthread_once_t g_knobs_once = PTHREAD_ONCE_INIT;
+
+static void knobs_from_environment() {
+  for (int k = 0; k < KNOB_COUNT; ++k) {
+    const char* e = getenv(kKnobNames[k]);
+    g_knobs[k] = (e && *e) ? atoi(e) : kKnobUnset;
+  }
+}
+
+int knob(Knob k) {
+  pthread_once(&g_knobs_once, knobs_from_environment);
+  return __atomic_load_n(&g_knobs[k], __ATOMIC_RELAXED);
+}
+
 }  // namespace samfast
+
+extern "C" int samfast_bench_set_knob(const char* name, int value, int unset) {
+  using namespace samfast;
+  SF_REQUIRE(name, "bench_set_knob: null name");
+  pthread_once(&g_knobs_once, knobs_from_environment);
+  for (int k = 0; k < KNOB_COUNT; ++k)
+    if (strcmp(name, kKnobNames[k]) == 0) {
+      __atomic_store_n(&g_knobs[k], unset ? kKnobUnset : value, __ATOMIC_RELAXED);
+      return SAMFAST_OK;
+    }
+  SF_FAIL(SAMFAST_E_INVALID, "bench_set_knob: unknown knob %s", name);
+}
 
 extern "C" int samfast_version(void) { return SAMFAST_VERSION; }
 extern "C" const char* samfast_arch(void) { return "gfx950"; }

@@ -943,8 +943,8 @@ static int launch_hd(const AttnArgs& a, bool global_path, hipStream_t stream) {
     // 256 queries per workgroup when that still gives every CU several workgroups
     // (SAMFAST_ATTN_WAVES=4 / 8 overrides the choice where the shape allows it)
     const int64_t wg8 = (int64_t)a.B * a.nH * (a.N / 256);
-    const char* force = getenv("SAMFAST_ATTN_WAVES");
-    const bool want8 = force ? atoi(force) == 8 : wg8 >= 1024;
+    const int force = knob(KNOB_ATTN_WAVES);
+    const bool want8 = force != kKnobUnset ? force == 8 : wg8 >= 1024;
     if (a.N % 256 == 0 && want8) launch(std::integral_constant<int, 8>{});
     else launch(std::integral_constant<int, 4>{});
     return check_launch("attn_global_kernel");

@@ -49,6 +49,7 @@
 // quant_rowwise.hip, one wavefront per row, rows double-buffered) over them, then puts the
 // counter back to zero for the next launch.  The other workgroup resident on the CU keeps the
 // matrix pipe busy meanwhile.
+#include "gemm_i8_shared.hpp"
 #include "quant_row.hpp"
 #include <pthread.h>
 #include <stdlib.h>
@@ -59,38 +60,6 @@
 #pragma clang fp contract(off)
 
 namespace samfast {
-
-constexpr int GBN = 256, GBK = 64;
-constexpr int GLD = GBK;  // LDS row, bytes (unpadded; chunks are XOR-swizzled instead)
-
-enum { EPI_I32 = 0, EPI_SCALE_BIAS_BF16 = 1, EPI_GELU_BF16 = 2, EPI_RESIDUAL_BF16 = 3 };
-
-struct GemmArgs {
-  const int8_t* x;
-  const int8_t* w;
-  void* out;
-  const float* sx;
-  const float* sw;
-  const float* bias;
-  int64_t ldo;
-  int M, N, K;
-  int tiles_m, tiles_n;
-  int group_m;     // row tiles per scheduling group
-  int stream_out;  // outputs without residual that exceed the 256 MB last-level cache
-  int row_pitch;            // bytes between consecutive rows of X / W: K (row-major) or 64 (K-block major)
-  int64_t x_kstep, w_kstep; // bytes between consecutive 64-byte k tiles: 64, or rows * 64
-  const unsigned short* residual;  // EPI_RESIDUAL: (rows, N) bf16, row stride ld_res
-  int64_t ld_res;
-  const int32_t* dst_row;          // EPI_RESIDUAL: output row per GEMM row, -1 = drop; may be null
-  // quantiser of the output rows (kernels with TAILN > 0)
-  int32_t* tile_counters;          // one per row tile; zero before the launch and again after it
-  int8_t* yq;                      // codes of the (LayerNorm of the) output rows, layout yq_kb64
-  float* sy;                       // their scales
-  const unsigned short* ln_gamma;  // TAILLN: LayerNorm weight / bias (N bf16 values each)
-  const unsigned short* ln_beta;
-  float ln_eps;
-  int yq_kb64;
-};
 
 // Epilogue shared by the kernels: the lane owns 4 adjacent output columns of each of
 // its 16*TM rows (MFMA tile i, register r -> row i*32 + 8*(r/4) + 4*lh + r%4).
@@ -366,12 +335,6 @@ SF_DEVICE void gemm_quant_tail(const GemmArgs& a, int m0, int tile_m, int tid, i
   }
   if (tid == 0) a.tile_counters[tile_m] = 0;  // the next launch finds the counter at zero
 }
-
-// 16-byte chunk c of LDS row r lives at chunk position c ^ lds_swizzle(r).  With it the
-// operand reads (one chunk of 8 / 16 consecutive rows per LDS cycle) and the tile writes
-// (4 chunks of 2 / 4 consecutive rows per cycle) both touch every bank once, whether the
-// LDS cycles through 128 or 256 bytes.
-SF_DEVICE int lds_swizzle(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
 
 template <int EPI, int TM, bool GENERIC, int TAILN = 0, bool TAILLN = false>
 __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArgs a) {
@@ -924,8 +887,7 @@ static bool tail_built(int epi, bool ln, int N) {
 
 // whether gemm_common would run `tail` inside the GEMM for this call
 static bool tail_fusable(int epi, const GemmTail& t, int N, int K, const int32_t* dst_row) {
-  const char* force = getenv("SAMFAST_GEMM_TM");
-  return K / GBK >= 4 && !(force && atoi(force) == 4) && !dst_row && tail_built(epi, t.gamma != nullptr, N);
+  return K / GBK >= 4 && knob(KNOB_GEMM_TM) != 4 && !dst_row && tail_built(epi, t.gamma != nullptr, N);
 }
 
 static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t* wq,
@@ -968,9 +930,8 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   }
   a.residual = reinterpret_cast<const unsigned short*>(residual);
   a.ld_res = ld_res; a.dst_row = dst_row;
-  const char* force = getenv("SAMFAST_GEMM_TM");  // tuning aid: 2 or 4
   const bool generic_k = K / GBK < 4;  // fewer k tiles than LDS stages
-  const int tm = generic_k ? 2 : (force && atoi(force) == 4 ? 4 : 2);
+  const int tm = generic_k ? 2 : (knob(KNOB_GEMM_TM) == 4 ? 4 : 2);  // tuning aid: 2 or 4
   const int bm = 64 * tm;
   a.tiles_m = (int)((M + bm - 1) / bm);
   a.tiles_n = (N + GBN - 1) / GBN;
@@ -990,16 +951,16 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   }
   const int64_t total = (int64_t)a.tiles_m * a.tiles_n;
   SF_REQUIRE(total < (1ll << 30), "gemm_i8: too many tiles");
+  // resident workgroups that walk a list of tiles each (SAMFAST_GEMM_PERSIST=1), where built
+  if (!tail && !generic_k && tm == 2 && gemm_i8_persist_covers(epi, a)) return gemm_i8_persist_launch(epi, a, stream);
   const unsigned int grid = (unsigned int)(((total + 7) / 8) * 8);
   const bool generic = generic_k;
   // the three-workgroups-per-CU form of the main kernel (SAMFAST_GEMM_WG3=0: two per CU)
-  const char* wg3 = getenv("SAMFAST_GEMM_WG3");
-  if (!tail && !generic && tm == 2 && epi != EPI_I32 && !(wg3 && atoi(wg3) == 0)) {
+  if (!tail && !generic && tm == 2 && epi != EPI_I32 && knob(KNOB_GEMM_WG3) != 0) {
     // 64 x 128 tiles when 128 x 256 ones would leave more than half of the 768 workgroup slots of
     // the GPU empty (SAMFAST_GEMM_TILE=64 / 128 forces either)
-    const char* ft = getenv("SAMFAST_GEMM_TILE");
-    const char* fb = getenv("SAMFAST_GEMM_SMALL_BELOW");  // tuning aid: the tile-count threshold
-    const bool small = ft ? atoi(ft) == 64 : total < (fb ? atoi(fb) : 384);
+    const int ft = knob(KNOB_GEMM_TILE);
+    const bool small = ft != kKnobUnset ? ft == 64 : total < knob_or(KNOB_GEMM_SMALL_BELOW, 384);
     if (small) {
       a.tiles_m = (int)((M + 63) / 64);
       a.tiles_n = (N + 127) / 128;
@@ -1124,6 +1085,9 @@ extern "C" int samfast_gemm_i8_fused_quant(const int8_t* xq, const float* sx, co
       set_error("gemm_i8_fused_quant: unknown epilogue %d", epilogue);
       return SAMFAST_E_INVALID;
   }
+  // the quantiser addresses yq with 32-bit lane offsets (the two-launch form checks the same limit)
+  SF_REQUIRE(M >= 0 && N > 0 && M * (int64_t)N < (1ll << 31),
+             "gemm_i8_fused_quant: outputs of 2^31 elements or more are not supported (M=%lld N=%d)", (long long)M, N);
   SF_REQUIRE((ln_gamma == nullptr) == (ln_beta == nullptr), "gemm_i8_fused_quant: gamma and beta go together");
   SF_REQUIRE(M == 0 || (yq && sy && tile_counters), "gemm_i8_fused_quant: null output or counter pointer");
   SF_REQUIRE(yq_layout == SAMFAST_LAYOUT_ROWMAJOR || (yq_layout == SAMFAST_LAYOUT_KB64 && N % 64 == 0),
@@ -1199,6 +1163,9 @@ extern "C" int samfast_gemm_i8_fused_quant_noalloc(const int8_t* xq, const float
              "gemm_i8_fused_quant_noalloc: M=%lld needs %lld row-tile counters, the built-in workspace holds %d "
              "(at most %lld rows); use samfast_gemm_i8_fused_quant with a workspace of your own",
              (long long)M, (long long)tiles, kNoAllocMaxTiles, (long long)kNoAllocMaxTiles * 128);
+  SF_REQUIRE(N > 0 && M * (int64_t)N < (1ll << 31),
+             "gemm_i8_fused_quant_noalloc: outputs of 2^31 elements or more are not supported (M=%lld N=%d)",
+             (long long)M, N);
   int32_t* counters = nullptr;
   const int rc = scratch_of_current_device(&counters);
   if (rc != SAMFAST_OK) return rc;

@@ -13,6 +13,7 @@
 // a condition on the data that the compiler cannot decide, so the arithmetic stays, and that in
 // practice never holds, so the kernel writes nothing.
 #include "samfast_internal.hpp"
+#include "samfast_bench.h"
 
 namespace samfast {
 
@@ -127,6 +128,9 @@ extern "C" int samfast_bench_mfma_valu_overlap(int vector_kind, const void* oper
   SF_REQUIRE(workgroups > 0 && workgroups <= (1 << 20) && mfma_rounds >= 0 && mfma_rounds <= (1 << 24) &&
                  vector_rounds >= 0 && vector_rounds <= (1 << 24),
              "bench_mfma_valu_overlap: bad workgroup or round count");
+  // a launch stays below about a second of GPU time
+  SF_REQUIRE((int64_t)workgroups * ((int64_t)mfma_rounds + vector_rounds) <= (1ll << 27),
+             "bench_mfma_valu_overlap: workgroups * rounds must not exceed 2^27");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const u32x4* ops = reinterpret_cast<const u32x4*>(operands);
   if (vector_kind == 0)
@@ -145,6 +149,8 @@ extern "C" int samfast_bench_mfma_ceiling(int instruction, const void* operands,
   SF_REQUIRE(operands && scratch_out && aligned16(operands), "bench_mfma_ceiling: null or unaligned buffer");
   SF_REQUIRE(workgroups > 0 && workgroups <= (1 << 20) && iters > 0 && iters <= (1 << 24),
              "bench_mfma_ceiling: bad workgroup or iteration count");
+  // a launch stays below about a second of GPU time
+  SF_REQUIRE((int64_t)workgroups * iters <= (1ll << 27), "bench_mfma_ceiling: workgroups * iters must not exceed 2^27");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const u32x4* ops = reinterpret_cast<const u32x4*>(operands);
   if (instruction == 0)

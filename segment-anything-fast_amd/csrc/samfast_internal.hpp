@@ -22,6 +22,25 @@ void set_error(const char* fmt, ...);
 
 int check_launch(const char* what);
 
+// Tuning knobs: each is an environment variable read ONCE (at the first query of any knob), after
+// which samfast_bench_set_knob (include/samfast_bench.h) is the only way to change it.
+enum Knob {
+  KNOB_GEMM_TM,           // SAMFAST_GEMM_TM: 4 = 256 x 256 tiles in the two-per-CU kernel
+  KNOB_GEMM_WG3,          // SAMFAST_GEMM_WG3: 0 = two workgroups per CU instead of three
+  KNOB_GEMM_TILE,         // SAMFAST_GEMM_TILE: 64 / 128 forces the small / large tile of the three-per-CU kernel
+  KNOB_GEMM_SMALL_BELOW,  // SAMFAST_GEMM_SMALL_BELOW: tile count below which the small tile is taken
+  KNOB_GEMM_PERSIST,      // SAMFAST_GEMM_PERSIST: 0 off, 1 where it pays, 2 wherever it is built
+  KNOB_GEMM_SPLITK,       // SAMFAST_GEMM_SPLITK: 0 off, 1 where it pays (launches that leave the GPU half empty)
+  KNOB_ATTN_WAVES,        // SAMFAST_ATTN_WAVES: 4 / 8 wavefronts per global-attention workgroup
+  KNOB_COUNT
+};
+constexpr int kKnobUnset = INT32_MIN;
+int knob(Knob k);                      // kKnobUnset when neither the environment nor a setter gave a value
+static inline int knob_or(Knob k, int dflt) {
+  const int v = knob(k);
+  return v == kKnobUnset ? dflt : v;
+}
+
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---- vector types -------------------------------------------------------------

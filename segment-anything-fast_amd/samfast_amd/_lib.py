@@ -1,4 +1,5 @@
-"""ctypes binding of libsamfast.so (the C ABI declared in include/samfast.h).
+"""ctypes binding of libsamfast.so (the C ABI declared in include/samfast.h, plus the
+measurement aids of include/samfast_bench.h).
 
 The library is looked up next to this package (lib/libsamfast.so, built in-tree
 by segment-anything-fast_amd/build.py).  There is no fallback: if it is missing
@@ -47,6 +48,11 @@ _SIGNATURES = {
     "samfast_gemm_i8_sparse24_fused": (
         _i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _i32,
                _ptr, _i64, _i32, _ptr]),
+}
+
+# include/samfast_bench.h: measurement and tuning aids, not part of the path's ABI
+_BENCH_SIGNATURES = {
+    "samfast_bench_set_knob": (_i32, [ctypes.c_char_p, _i32, _i32]),
     "samfast_bench_mfma_ceiling": (_i32, [_i32, _ptr, _i32, _i32, ctypes.POINTER(_i64), _ptr, _ptr]),
     "samfast_bench_mfma_valu_overlap": (_i32, [_i32, _ptr, _i32, _i32, _i32, _ptr, _ptr]),
 }
@@ -55,6 +61,7 @@ EPILOGUE_NONE, EPILOGUE_GELU, EPILOGUE_RESIDUAL = 0, 1, 2
 LAYOUT_ROWMAJOR, LAYOUT_KB64 = 0, 1
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+BENCH_SYMBOLS = tuple(_BENCH_SIGNATURES)
 
 
 def lib_path() -> Path:
@@ -71,7 +78,7 @@ def load() -> ctypes.CDLL:
                 f"samfast: {path} not found - build it with "
                 "`python segment-anything-fast_amd/build.py` (there is no fallback path)")
         lib = ctypes.CDLL(str(path))
-        for name, (restype, argtypes) in _SIGNATURES.items():
+        for name, (restype, argtypes) in {**_SIGNATURES, **_BENCH_SIGNATURES}.items():
             fn = getattr(lib, name)
             fn.restype = restype
             fn.argtypes = argtypes
@@ -83,3 +90,25 @@ def check(code: int, what: str) -> None:
     if code != 0:
         msg = load().samfast_last_error().decode("utf-8", "replace")
         raise RuntimeError(f"samfast: {what} failed ({code}): {msg}")
+
+
+class knobs:
+    """Context manager that sets kernel-variant knobs (include/samfast_bench.h) for the calls inside
+    it and puts them back to "not given" afterwards: `with knobs(SAMFAST_GEMM_WG3=0): ...`.  The
+    library reads the environment variables of the same names once, at its first launch, so
+    changing os.environ later has no effect; this is the way to switch variants inside a process."""
+
+    def __init__(self, **values: int) -> None:
+        self.values = values
+
+    def __enter__(self):
+        lib = load()
+        for name, value in self.values.items():
+            check(lib.samfast_bench_set_knob(name.encode(), int(value), 0), "bench_set_knob")
+        return self
+
+    def __exit__(self, *exc):
+        lib = load()
+        for name in self.values:
+            check(lib.samfast_bench_set_knob(name.encode(), 0, 1), "bench_set_knob")
+        return False

@@ -14,23 +14,60 @@ import torch.nn as nn
 ROOT = Path(__file__).resolve().parents[1]
 
 
-def _header_functions():
-    text = (ROOT / "include" / "samfast.h").read_text()
+def _header_functions(header="samfast.h"):
+    text = (ROOT / "include" / header).read_text()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(samfast_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():
+    """include/samfast.h is the path's boundary; include/samfast_bench.h holds the measurement
+    aids.  The library exports exactly what the two declare and the Python binding mirrors both."""
     from samfast_amd import _lib
     names = _header_functions()
     assert len(names) >= 8
+    assert not [n for n in names if n.startswith("samfast_bench_")]
+    bench = _header_functions("samfast_bench.h")
+    assert bench and all(n.startswith("samfast_bench_") for n in bench)
     lib = ctypes.CDLL(str(_lib.lib_path()))
-    for n in names:
+    for n in names + bench:
         assert hasattr(lib, n), n
     assert sorted(_lib.EXPORTED_SYMBOLS) == names
+    assert sorted(_lib.BENCH_SYMBOLS) == bench
     loaded = _lib.load()
     assert loaded.samfast_version() == 1
     assert loaded.samfast_arch() == b"gfx950"
+
+
+def test_knobs_are_named_and_bounded_without_gpu():
+    """The variant knobs take the documented names only; the bare matrix-instruction loops refuse
+    launches that would hold the GPU for more than about a second (checked before any launch)."""
+    from samfast_amd import _lib
+    lib = _lib.load()
+    assert lib.samfast_bench_set_knob(b"SAMFAST_GEMM_PERSIST", 1, 0) == 0
+    assert lib.samfast_bench_set_knob(b"SAMFAST_GEMM_PERSIST", 0, 1) == 0
+    assert lib.samfast_bench_set_knob(b"SAMFAST_NO_SUCH_KNOB", 1, 0) == -1
+    assert b"unknown knob" in lib.samfast_last_error()
+    buf = ctypes.create_string_buffer(65536)
+    p = ctypes.addressof(buf)
+    p += (-p) % 16
+    assert lib.samfast_bench_mfma_ceiling(0, p, 1 << 20, 1 << 24, None, p, None) == -1
+    assert b"2^27" in lib.samfast_last_error()
+    assert lib.samfast_bench_mfma_valu_overlap(0, p, 1 << 12, 1 << 20, 0, p, None) == -1
+    assert b"2^27" in lib.samfast_last_error()
+
+
+def test_fused_quant_gemm_refuses_outputs_its_quantiser_cannot_address():
+    """lin1-shaped call with M * N >= 2^31: the in-kernel quantiser's 32-bit offsets would wrap, so
+    the entry point (and its allocation-free form) refuses before anything is launched."""
+    from samfast_amd import _lib
+    lib = _lib.load()
+    M, N, K = 900000, 5120, 1280  # M * K < 2^31 <= M * N
+    args = [None, None, None, None, None, None, N, M, N, K, 0, 1, None, 0, 1, None, None, 0.0, None, None, 1]
+    assert lib.samfast_gemm_i8_fused_quant(*args, None, None) == -1
+    assert b"2^31" in lib.samfast_last_error()
+    assert lib.samfast_gemm_i8_fused_quant_noalloc(*args, None) == -1
+    assert b"2^31" in lib.samfast_last_error()
 
 
 def test_empty_calls_are_no_ops_without_gpu():

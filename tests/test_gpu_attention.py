@@ -207,16 +207,16 @@ def test_rising_maximum_along_the_keys(gh, gw, hd, ramp):
 
 
 @pytest.mark.parametrize("hd,gh", [(80, 64), (64, 64), (80, 8)])
-def test_global_kernel_wave_count_variants_agree(monkeypatch, hd, gh):
+def test_global_kernel_wave_count_variants_agree(hd, gh):
     """The global kernel runs with 128 or 256 queries per workgroup (4 or 8 wavefronts); the choice
     follows the grid size and can be forced.  A query's arithmetic does not depend on it."""
-    from samfast_amd import ops
+    from samfast_amd import _lib, ops
     B, nH, gw = 1, 2, 64
     q, k, v, rph, rpw = (t.cuda() for t in attn_inputs(B, nH, gh, gw, hd, seed=5))
     outs = {}
     for waves in ("4", "8"):
-        monkeypatch.setenv("SAMFAST_ATTN_WAVES", waves)
-        outs[waves] = ops.attn_relpos(q, k, v, rph, rpw, (gh, gw)).clone()
+        with _lib.knobs(SAMFAST_ATTN_WAVES=int(waves)):
+            outs[waves] = ops.attn_relpos(q, k, v, rph, rpw, (gh, gw)).clone()
     torch.cuda.synchronize()
     assert torch.equal(outs["4"], outs["8"])
     ref = _oracle_tables(q.cpu(), k.cpu(), v.cpu(), rph.cpu(), rpw.cpu(), (gh, gw))

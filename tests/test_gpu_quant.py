@@ -481,7 +481,7 @@ def test_gemm_with_output_quantiser_in_place_residual():
 
 @pytest.mark.parametrize("M,N,K,epi", [(300, 1280, 1280, "residual"), (1000, 3840, 1280, "none"),
                                        (513, 5120, 1280, "gelu"), (260, 1280, 5120, "residual_scatter")])
-def test_gemm_two_and_three_workgroups_per_cu_agree(monkeypatch, M, N, K, epi):
+def test_gemm_two_and_three_workgroups_per_cu_agree(M, N, K, epi):
     """The main GEMM kernel exists in three forms - three workgroups per CU with 128 x 256 tiles
     (single-buffered fragments, two LDS stages, epilogue staged 64 rows at a time; the default), the
     same with 64 x 128 tiles (small launches, SAMFAST_GEMM_TILE=64) and two per CU
@@ -506,17 +506,60 @@ def test_gemm_two_and_three_workgroups_per_cu_agree(monkeypatch, M, N, K, epi):
             kw["dst_row"] = perm.cuda()
     outs = []
     # three per CU with 128 x 256 tiles, three (or more) per CU with 64 x 128 tiles, two per CU
-    for wg3, tile in (("1", "128"), ("1", "64"), ("0", "128")):
-        monkeypatch.setenv("SAMFAST_GEMM_WG3", wg3)
-        monkeypatch.setenv("SAMFAST_GEMM_TILE", tile)
-        out = torch.zeros_like(kw["residual"]) if "residual" in kw else None
-        outs.append(ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L, out=out, **kw).clone())
+    for wg3, tile in ((1, 128), (1, 64), (0, 128)):
+        with _lib.knobs(SAMFAST_GEMM_WG3=wg3, SAMFAST_GEMM_TILE=tile):
+            out = torch.zeros_like(kw["residual"]) if "residual" in kw else None
+            outs.append(ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L, out=out, **kw).clone())
     torch.cuda.synchronize()
     assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
     assert torch.equal(outs[1].view(torch.int16), outs[2].view(torch.int16))
 
 
-def test_gelu_epilogue_all_bf16_inputs(monkeypatch):
+@pytest.mark.parametrize("M,N,K,epi", [
+    (16384, 3840, 1280, "none"),   # 1920 tiles on 512 resident workgroups: lists of 3 and 4 tiles
+    (16384, 5120, 1280, "gelu"),
+    (8192, 2304, 768, "none"),     # 12 k tiles: the form whose stores leave over 8 iterations
+    (8320, 3072, 1024, "gelu"),
+    (1024, 1280, 5120, "none"),    # fewer tiles than workgroups: one tile each, 80 k tiles
+    (65536, 3840, 1280, "none"),   # the qkv Linear at full size: streaming stores, 15 tiles per workgroup
+])
+def test_gemm_persistent_form_agrees(M, N, K, epi):
+    """The persistent form of the 128 x 256 kernel (resident workgroups that walk a list of tiles,
+    the previous tile's output leaving inside the next tile's K loop) against the default form, bit
+    for bit over the whole output, and against the oracle on a sample of rows."""
+    from samfast_amd import _lib, ops
+    print(f"case persistent gemm M={M} N={N} K={K} {epi}", flush=True)
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16)
+    x[torch.randperm(M, generator=g)[:max(1, M // 1000)]] *= 20.0
+    w = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    bias = (torch.randn((N,), generator=g) * 0.02).cuda()
+    L = _lib.LAYOUT_KB64
+    xq, sx = ops.quant_rowwise(x.cuda(), L)
+    wq, sw = ops.quant_rowwise(w.cuda(), L)
+    code = {"none": _lib.EPILOGUE_NONE, "gelu": _lib.EPILOGUE_GELU}[epi]
+    want = ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L)
+    with _lib.knobs(SAMFAST_GEMM_PERSIST=2):
+        got = ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L)
+        again = ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(again.view(torch.int16), want.view(torch.int16))
+    # the oracle on rows spread over the first, a middle and the last row tile
+    rows = torch.cat([torch.arange(0, 3), torch.arange(M // 2 - 1, M // 2 + 2), torch.arange(M - 3, M)])
+    xq_r, sx_r = orq.quantize_rows_absmax(x[rows])
+    wq_r, sw_r = orq.quantize_rows_absmax(w)
+    acc = orq.int8_gemm_i32(xq_r, wq_r)
+    ref = orq.scale_bias_epilogue(acc, sx_r, sw_r, bias.cpu())
+    sample = got[rows.cuda()].cpu()
+    if epi == "none":
+        assert torch.equal(sample.view(torch.int16), ref.view(torch.int16))
+    else:
+        act = torch.nn.functional.gelu(ref.float()).to(torch.bfloat16).float()
+        assert torch.allclose(sample.float(), act, rtol=2 ** -7, atol=1e-6)  # one bf16 step
+
+
+def test_gelu_epilogue_all_bf16_inputs():
     """Every bf16 bit pattern through the GELU epilogue.  Zero weights and bias[n] = the bf16
     value with bits n make column n of the Linear output that value, so one launch evaluates the
     activation on all 65 536 inputs.  The three forms of the kernel (128 x 256 and 64 x 128 tiles
@@ -533,11 +576,10 @@ def test_gelu_epilogue_all_bf16_inputs(monkeypatch):
         sx = torch.ones((M,), dtype=torch.float32).cuda()
         wq = torch.zeros((N, K), dtype=torch.int8).cuda()
         sw = torch.ones((N,), dtype=torch.float32).cuda()
-        for name, wg3, tile in (("large", "1", "128"), ("small", "1", "64"), ("two", "0", "128")):
-            monkeypatch.setenv("SAMFAST_GEMM_WG3", wg3)
-            monkeypatch.setenv("SAMFAST_GEMM_TILE", tile)
-            y = ops.gemm_i8_fused(xq, sx, wq, sw, bias, _lib.EPILOGUE_GELU)
-            torch.cuda.synchronize()
+        for name, wg3, tile in (("large", 1, 128), ("small", 1, 64), ("two", 0, 128)):
+            with _lib.knobs(SAMFAST_GEMM_WG3=wg3, SAMFAST_GEMM_TILE=tile):
+                y = ops.gemm_i8_fused(xq, sx, wq, sw, bias, _lib.EPILOGUE_GELU)
+                torch.cuda.synchronize()
             assert torch.equal(y[0].view(torch.int16), y[M - 1].view(torch.int16))
             outs[(K, name)] = y[0].cpu()
     want = outs[(256, "two")]
