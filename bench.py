@@ -302,9 +302,10 @@ def gemm_variants(batch=16, width=1280):
     dev = torch.device("cuda:0")
     M = batch * 4096
     g = torch.Generator(device="cuda").manual_seed(11)
-    variants = [("three_workgroups_per_cu (default)", {}),
-                ("two_workgroups_per_cu", {"SAMFAST_GEMM_WG3": 0}),
-                ("persistent (where built, else the default)", {"SAMFAST_GEMM_PERSIST": 1})]
+    variants = [("three_workgroups_per_cu", {"SAMFAST_GEMM_PERSIST": 0}),
+                ("two_workgroups_per_cu", {"SAMFAST_GEMM_PERSIST": 0, "SAMFAST_GEMM_WG3": 0}),
+                ("persistent, all workgroups start together", {"SAMFAST_GEMM_PERSIST": 2, "SAMFAST_GEMM_PERSIST_SKEW": 0}),
+                ("persistent, every second workgroup starts a tile late", {"SAMFAST_GEMM_PERSIST": 2})]
     shapes = [("qkv", 3 * width, width, _lib.EPILOGUE_NONE), ("proj", width, width, _lib.EPILOGUE_RESIDUAL),
               ("lin1", 4 * width, width, _lib.EPILOGUE_GELU), ("lin2", width, 4 * width, _lib.EPILOGUE_RESIDUAL)]
     res = {"what": f"gemm_i8 at M={M}, us per launch (10 back to back) and TOP/s, per variant knob, on "

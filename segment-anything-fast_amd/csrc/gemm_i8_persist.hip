@@ -16,7 +16,14 @@
 // operations complete in issue order, so "tile kt+1 has landed" stays a vmcnt threshold that
 // counts the younger loads and stores exactly.
 //
-// Covered: scale + bias and GELU epilogues on full tiles (M % 128 == 0, N % 256 == 0, K >= 768).
+// Residual epilogue: the residual values of the rows that leave with the conversion (and of the first
+// held stores) are requested in the tile's last iteration, ahead of that iteration's tile loads, so a
+// vmcnt wait that still leaves those tile loads in flight covers them; every later held store gets
+// its residual one iteration ahead, again requested before the stores and tile loads it must not wait
+// for.  Output and residual may be the same buffer: a lane reads a location before it writes it.
+//
+// Covered: scale + bias, GELU and residual (no row scatter) epilogues on full tiles (M % 128 == 0,
+// N % 256 == 0, K >= 768).
 // Arithmetic, operand layouts in LDS and the tile -> XCD mapping are those of gemm_i8_kernel, and
 // the results are bit-equal.
 #include "gemm_i8_shared.hpp"
@@ -30,6 +37,9 @@
 
 namespace samfast {
 
+#ifndef PERSIST_MIN_WG
+#define PERSIST_MIN_WG 2
+#endif
 constexpr int PBM = 128, PBN = 256;
 constexpr int PNST = 3;                           // LDS operand stages
 constexpr int PSTAGE = (PBM + PBN) * GLD;         // 24 KB
@@ -40,9 +50,17 @@ constexpr int PSC_LOADS = 3;                      // scale loads per wavefront a
 template <int V>
 using IC = std::integral_constant<int, V>;
 
+// compile-time shape of one k iteration of gemm_i8_persist_kernel (see `iteration` there)
+template <bool ZERO_, bool CONV_, int S0_, int NSTORE_, int D_, bool RFIRST_, bool SC_, bool ISSUE_, bool NEXT_, int THRESH_>
+struct PersistIter {
+  static constexpr bool ZERO = ZERO_, CONV = CONV_, RFIRST = RFIRST_, SC = SC_, ISSUE = ISSUE_, NEXT = NEXT_;
+  static constexpr int S0 = S0_, NSTORE = NSTORE_, D = D_, THRESH = THRESH_;
+};
+
 template <int EPI, int DI, int IMM, bool NT>
-__global__ __launch_bounds__(256, 2) void gemm_i8_persist_kernel(GemmArgs a) {
-  static_assert(EPI == EPI_SCALE_BIAS_BF16 || EPI == EPI_GELU_BF16, "epilogues built");
+__global__ __launch_bounds__(256, PERSIST_MIN_WG) void gemm_i8_persist_kernel(GemmArgs a) {
+  static_assert(EPI == EPI_SCALE_BIAS_BF16 || EPI == EPI_GELU_BF16 || EPI == EPI_RESIDUAL_BF16, "epilogues built");
+  constexpr bool RES = EPI == EPI_RESIDUAL_BF16;
   static_assert((32 - IMM) % DI == 0, "the held stores of a wavefront are spread evenly over DI iterations");
   constexpr int NS = (32 - IMM) / DI;  // stores per drain iteration
   __shared__ __attribute__((aligned(16))) unsigned char lds[PNST * PSTAGE + 2 * PSC_BYTES];
@@ -92,6 +110,7 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_persist_kernel(GemmArgs a) {
         const int wrow = (sl & 128) + (sl & 31) * 4 + ((sl & 127) >> 5);
         dma_off[i] = (unsigned int)((n0 + wrow) * a.row_pitch + chunk16);
       }
+      asm volatile("" : "+v"(dma_off[i]));  // a 32-bit value from here on (not a widened 64-bit product)
     }
   };
   auto dma_issue = [&](int kt, int stage_off) __attribute__((always_inline)) {
@@ -151,38 +170,22 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_persist_kernel(GemmArgs a) {
   // i*32 + 8*(r/4) + 4*lh + r%4); held[i][r] keeps them as two packed bf16 pairs.
   u32x2 held[2][16];
   f32x4 swv, bv4;
+  // residual epilogue: values of the IMM rows that leave with the conversion plus the first NS held
+  // stores (requested in the tile's last iteration), and of the held stores of the iterations
+  // d (slot d & 1), each requested one iteration ahead
+  u32x2 res_first[RES ? IMM + NS : 1];
+  u32x2 res_ring[2][RES ? NS : 1];
+  auto add_residual = [&](u32x2& val, const u32x2& r) __attribute__((always_inline)) {
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+      // bf16 add of the bf16-rounded Linear output and the residual stream
+      val[c] = pack_bf16x2(bf16_lo_to_f32(val[c]) + bf16_lo_to_f32(r[c]),
+                           bf16_hi_to_f32(val[c]) + bf16_hi_to_f32(r[c]));
+  };
   auto convert_begin = [&](const unsigned char* sc) __attribute__((always_inline)) {
     swv = *reinterpret_cast<const f32x4*>(sc + 512 + (wn * 128 + 4 * lr) * 4);
     const f32x4 z = {0.f, 0.f, 0.f, 0.f};
     bv4 = a.bias ? *reinterpret_cast<const f32x4*>(sc + 1536 + (wn * 128 + 4 * lr) * 4) : z;
-  };
-  auto convert_half = [&](int i, const unsigned char* sc) __attribute__((always_inline)) {
-    f32x4 sxv[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g)
-      sxv[g] = *reinterpret_cast<const f32x4*>(sc + (wm * 64 + i * 32 + 8 * g + 4 * lh) * 4);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float s = sxv[r >> 2][r & 3];
-      float y[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // three separately rounded fp32 operations (no fused multiply-add)
-        float t = (float)acc[i][j][r] * s;
-        t = t * swv[j];
-        y[j] = t + bv4[j];
-      }
-      u32x2 o = {pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3])};
-      if (EPI == EPI_GELU_BF16) {
-        // activation of the bf16-rounded Linear output, as a separate GELU would see it
-        o[0] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[0])), gelu_erf(bf16_hi_to_f32(o[0])));
-        o[1] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[1])), gelu_erf(bf16_hi_to_f32(o[1])));
-      }
-      held[i][r] = o;
-      // keep the conversion narrow (four rows at a time): scheduled for parallelism it would hold
-      // all 64 values of a half as floats at once
-      if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);
-    }
   };
   // byte offset of the lane's first element inside an output tile; rows are added as uniform offsets
   const unsigned int voff = (unsigned int)(((wm * 64 + 4 * lh) * a.ldo + wn * 128 + 4 * lr) * 2);
@@ -206,6 +209,52 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_persist_kernel(GemmArgs a) {
     else *dst = held[i][r];
   };
 
+  auto convert_half = [&](int i, const unsigned char* sc, bool store_now) __attribute__((always_inline)) {
+    f32x4 sxv[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      sxv[g] = *reinterpret_cast<const f32x4*>(sc + (wm * 64 + i * 32 + 8 * g + 4 * lh) * 4);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float s = sxv[r >> 2][r & 3];
+      float y[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // three separately rounded fp32 operations (no fused multiply-add)
+        float t = (float)acc[i][j][r] * s;
+        t = t * swv[j];
+        y[j] = t + bv4[j];
+      }
+      u32x2 o = {pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3])};
+      if (EPI == EPI_GELU_BF16) {
+        // activation of the bf16-rounded Linear output, as a separate GELU would see it
+        o[0] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[0])), gelu_erf(bf16_hi_to_f32(o[0])));
+        o[1] = pack_bf16x2(gelu_erf(bf16_lo_to_f32(o[1])), gelu_erf(bf16_hi_to_f32(o[1])));
+      }
+      if (RES && i == 0) add_residual(o, res_first[r]);  // these rows leave at once, residual included
+      held[i][r] = o;
+      if (store_now && i * 16 + r < IMM) store_piece(i * 16 + r);  // (its registers are free again at once)
+      // keep the conversion narrow (four rows at a time): scheduled for parallelism it would hold
+      // all 64 values of a half as floats at once
+      if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // residual values of store piece s of the tile whose output is converted next
+  const unsigned int voff_res = (unsigned int)(((wm * 64 + 4 * lh) * a.ld_res + wn * 128 + 4 * lr) * 2);
+  const unsigned short* prev_res = nullptr;  // residual + m0 * ld_res + n0 of that tile
+  auto residual_piece = [&](int s) __attribute__((always_inline)) {
+    const int i = s >> 4, r = s & 15;
+    unsigned int pitch = (unsigned int)a.ld_res * 2u;
+    asm volatile("" : "+s"(pitch));
+    const unsigned char* p = reinterpret_cast<const unsigned char*>(prev_res) +
+                             (unsigned int)(i * 32 + 8 * (r >> 2) + (r & 3)) * pitch;
+    asm volatile("" : "+s"(p));
+    unsigned int off = voff_res;
+    asm volatile("" : "+v"(off));
+    typedef __attribute__((address_space(1))) const u32x2* gsrc_t;
+    return *(gsrc_t)((gstore_t)(uintptr_t)p + off);
+  };
+
   // s_waitcnt immediate: vmcnt in bits 3:0 and 15:14 ("at most n operations still in flight"),
   // expcnt 6:4 = 7 (no wait), lgkmcnt 11:8 = 0 (all of this wave's LDS reads done)
   auto wait_imm = [](int n) constexpr { return 0x0070 | (n & 15) | ((n >> 4) << 14); };
@@ -213,29 +262,37 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_persist_kernel(GemmArgs a) {
   int st[PNST];  // st[j] = LDS offset of the stage holding k tile (current + j); uniform, rotated
   const unsigned char* conv_sc = lds + PNST * PSTAGE;  // scale buffer of the tile whose output is converted next
 
-  // One k iteration.  ZERO: first iteration of a tile (accumulators start at zero); CONV: the previous
-  // tile's accumulators are converted first; stores S0 .. S0+NSTORE-1 of the held output go out after
-  // the barrier; SC: the next tile's scales are requested (into scale buffer sc_buf) before the tile
-  // loads; ISSUE: k tile ld_kt is requested into the stage freed at the barrier; NEXT: a following k
-  // tile exists (of this tile or the next); THRESH: operations younger than the loads of the k tile
-  // needed next, i.e. what may stay in flight across the barrier.
-  auto iteration = [&](int ld_kt, int sc_m0, int sc_n0, int sc_buf, auto c_zero, auto c_conv, auto c_s0,
-                       auto c_nstore, auto c_sc, auto c_issue, auto c_next, auto c_thresh) __attribute__((always_inline)) {
-    constexpr bool ZERO = decltype(c_zero)::value != 0, CONV = decltype(c_conv)::value != 0;
-    constexpr int S0 = decltype(c_s0)::value, NSTORE = decltype(c_nstore)::value;
-    constexpr bool SC = decltype(c_sc)::value != 0, ISSUE = decltype(c_issue)::value != 0;
-    constexpr bool NEXT = decltype(c_next)::value != 0;
-    constexpr int THRESH = decltype(c_thresh)::value;
+  // One k iteration; F carries its compile-time shape:
+  //   ZERO    first iteration of a tile, accumulators start at zero;
+  //   CONV    the previous tile's accumulators are converted first (implies ZERO), IMM stores leave;
+  //   S0, NSTORE  held stores S0 .. S0+NSTORE-1 go out after the barrier, ahead of the tile loads;
+  //   D       index of a drain iteration (residual epilogue: which residual ring slot it uses);
+  //   RFIRST  residual epilogue: the residual values the next conversion needs are requested, ahead of
+  //           the tile loads (the tile's last iteration);
+  //   SC      the next tile's scales are requested (into scale buffer sc_buf) before the tile loads;
+  //   ISSUE   k tile ld_kt is requested into the stage freed at the barrier;
+  //   NEXT    a following k tile exists (of this tile or the next);
+  //   THRESH  operations younger than the loads of the k tile needed next, i.e. what may stay in
+  //           flight across the barrier.
+  auto iteration = [&](int ld_kt, int sc_m0, int sc_n0, int sc_buf, auto f) __attribute__((always_inline)) {
+    using F = decltype(f);
+    constexpr bool ZERO = F::ZERO, CONV = F::CONV, SC = F::SC, ISSUE = F::ISSUE, NEXT = F::NEXT, RFIRST = F::RFIRST;
+    constexpr int S0 = F::S0, NSTORE = F::NSTORE, THRESH = F::THRESH, D = F::D;
     if constexpr (CONV) {
+      // residual epilogue: the values requested in the last iteration have landed (its tile loads, the
+      // youngest operations in flight, need not have)
+      if constexpr (RES) __builtin_amdgcn_s_waitcnt(0x0F70 | PNLD);  // vmcnt <= PNLD, nothing else waited for
       // (the fences keep the zero-initialised matrix instructions of a row half behind the conversion
       // of that half: hoisted above it, old and new accumulators would be live together)
       convert_begin(conv_sc);
-      convert_half(0, conv_sc);
+      convert_half(0, conv_sc, true);  // the first IMM pieces leave as they are converted; the rest is held
       __builtin_amdgcn_sched_barrier(0);
+      // residual epilogue: the first fragments of this tile are read here rather than in the previous
+      // iteration (whose barrier made the k tile visible), so that they and the residual values the
+      // conversion consumes are not live together
+      if constexpr (RES) frags_at(st[0], 0, fa0, fb0);
       mma_zero_row(0, fa0, fb0);
-#pragma unroll
-      for (int s = 0; s < IMM; ++s) store_piece(s);  // these leave at once; the rest is held
-      convert_half(1, conv_sc);
+      convert_half(1, conv_sc, true);
       __builtin_amdgcn_sched_barrier(0);
       mma_zero_row(1, fa0, fb0);
       __builtin_amdgcn_sched_barrier(0);
@@ -259,28 +316,75 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_persist_kernel(GemmArgs a) {
     __builtin_amdgcn_s_waitcnt(wait_imm(THRESH));
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (RES && NSTORE > 0) {
+      // the next drain iteration's residual values first, then this iteration's stores: the wait for
+      // this iteration's values (requested an iteration ago, or with the conversion's) then covers
+      // nothing younger than them
+      constexpr bool MORE = S0 + 2 * NSTORE <= 32;  // another drain iteration follows
+      if constexpr (MORE) {
+#pragma unroll
+        for (int s = 0; s < NSTORE; ++s) res_ring[(D + 1) & 1][s] = residual_piece(S0 + NSTORE + s);
+      }
+      if constexpr (D > 0) {
+        constexpr int younger = NSTORE + PNLD + (MORE ? NSTORE : 0);
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (younger & 15) | ((younger >> 4) << 14));
+      }
+#pragma unroll
+      for (int s = 0; s < NSTORE; ++s) {
+        const int piece = S0 + s;
+        add_residual(held[piece >> 4][piece & 15], D == 0 ? res_first[IMM + s] : res_ring[D & 1][s]);
+      }
+    }
 #pragma unroll
     for (int s = 0; s < NSTORE; ++s) store_piece(S0 + s);
+    if constexpr (RES && RFIRST) {
+#pragma unroll
+      for (int s = 0; s < IMM + NS; ++s) res_first[s] = residual_piece(s);
+    }
     if constexpr (SC) scales_issue(sc_m0, sc_n0, sc_buf);
     if constexpr (ISSUE) dma_issue(ld_kt, st[0]);
     if constexpr (NEXT) frags_at(st[1], 0, fa0, fb0);
     mma(fa1, fb1);
+    if constexpr (!(RES && (NSTORE > 0 || RFIRST))) {
 #pragma unroll
-    for (int g = 0; g < 6; ++g) {
-      if constexpr (NEXT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      if (g < NSTORE) __builtin_amdgcn_sched_group_barrier(0x040, 1, 0);
-      if constexpr (SC) { if (g < PSC_LOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
-      if constexpr (ISSUE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      for (int g = 0; g < 6; ++g) {
+        if constexpr (NEXT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (g < NSTORE) __builtin_amdgcn_sched_group_barrier(0x040, 1, 0);
+        if constexpr (SC) { if (g < PSC_LOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
+        if constexpr (ISSUE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
     }
+    // The matrix instructions are pure values to the compiler: nothing but their operands ties them
+    // to this iteration, and instruction selection has been seen to sink three iterations' worth of
+    // them below the following barriers (their fragments then all live at once).  Passing the
+    // accumulators through an empty asm statement here pins every chain between two iterations.
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(acc[i][j]));
     __builtin_amdgcn_sched_barrier(0);
     const int t = st[0];
 #pragma unroll
     for (int j = 0; j + 1 < PNST; ++j) st[j] = st[j + 1];
     st[PNST - 1] = t;
   };
-  using Y = IC<1>;
-  using N = IC<0>;
+  // plain iteration: tile loads only, one k tile in flight across the barrier
+  using Plain = PersistIter<false, false, 0, 0, 0, false, false, true, true, PNLD>;
+
+  // Two resident workgroups that start in the same cycle run the same code on the same CU and tend
+  // to stay in step: both in their LDS reads, both at their barriers, both converting.  The
+  // workgroup whose first wavefront sits in an odd wave slot of its SIMD starts a.skew * 64 cycles late.
+  if (a.skew > 0) {
+    const unsigned int hw_id = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (3 << 11));  // HW_ID, WAVE_ID bits 3:0
+    int* flag = reinterpret_cast<int*>(lds + PNST * PSTAGE);
+    if (tid == 0) *flag = (int)(hw_id & 1u);
+    __syncthreads();
+    const int odd = __builtin_amdgcn_readfirstlane(*flag);
+    __syncthreads();
+    if (odd)
+      for (int i = 0; i < a.skew; ++i) __builtin_amdgcn_s_sleep(1);
+  }
 
   // ---- prologue: the first tile's scales and first three k tiles --------------------------------
   const int nk = a.K / GBK;
@@ -304,52 +408,67 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_persist_kernel(GemmArgs a) {
   auto tile_tail = [&](int ti) __attribute__((always_inline)) {
     // the output of this tile is converted at the top of the next one (or after the loop)
     prev_base = reinterpret_cast<const unsigned short*>(a.out) + (int64_t)m0 * a.ldo + n0;
+    if (RES) prev_res = a.residual + (int64_t)m0 * a.ld_res + n0;
     conv_sc = lds + PNST * PSTAGE + (ti & 1) * PSC_BYTES;
     const unsigned int nxt = ti + 1 < nt ? (unsigned int)(ti + 1) : (unsigned int)ti;
     tile_origin(first + nxt * per_x, m0, n0);
     set_dma(m0, n0);
-    iteration(0, m0, n0, (ti + 1) & 1, N{}, N{}, IC<0>{}, IC<0>{}, Y{}, Y{}, Y{}, IC<PNLD>{});
-    iteration(1, 0, 0, 0, N{}, N{}, IC<0>{}, IC<0>{}, N{}, Y{}, Y{}, IC<PNLD + PSC_LOADS>{});
-    iteration(2, 0, 0, 0, N{}, N{}, IC<0>{}, IC<0>{}, N{}, Y{}, Y{}, IC<PNLD>{});
+    iteration(0, m0, n0, (ti + 1) & 1, PersistIter<false, false, 0, 0, 0, false, true, true, true, PNLD>{});
+    iteration(1, 0, 0, 0, PersistIter<false, false, 0, 0, 0, false, false, true, true, PNLD + PSC_LOADS>{});
+    iteration(2, 0, 0, 0, PersistIter<false, false, 0, 0, 0, true, false, true, !RES, PNLD>{});
   };
 
   // ---- first tile: nothing to convert or store yet ----------------------------------------------
-  iteration(3, 0, 0, 0, Y{}, N{}, IC<0>{}, IC<0>{}, N{}, Y{}, Y{}, IC<PNLD>{});
-  for (int kt = 1; kt < nk - 3; ++kt) iteration(kt + 3, 0, 0, 0, N{}, N{}, IC<0>{}, IC<0>{}, N{}, Y{}, Y{}, IC<PNLD>{});
+  iteration(3, 0, 0, 0, PersistIter<true, false, 0, 0, 0, false, false, true, true, PNLD>{});
+  for (int kt = 1; kt < nk - 3; ++kt) iteration(kt + 3, 0, 0, 0, Plain{});
   tile_tail(0);
 
+  // residual values requested per drain iteration (they sit between the stores and tile loads that a
+  // threshold counts)
+  constexpr int NR = RES ? NS : 0;
   for (int ti = 1; ti < nt; ++ti) {
     // Iterations 0 .. DI-1 carry the previous tile's held stores, each ahead of its tile loads.
     // Younger than the k tile needed next: in iteration 0 one k tile and the IMM stores issued with
-    // the conversion; in iteration 1 those stores, iteration 0's and one k tile; from then on the
-    // stores of the iteration before and one k tile.
-    iteration(3, 0, 0, 0, Y{}, Y{}, IC<IMM>{}, IC<NS>{}, N{}, Y{}, Y{}, IC<PNLD + IMM>{});
-    iteration(4, 0, 0, 0, N{}, N{}, IC<IMM + NS>{}, IC<NS>{}, N{}, Y{}, Y{}, IC<PNLD + IMM + NS>{});
+    // the conversion; in iteration 1 those stores, iteration 0's (and the residual values requested
+    // with them) and one k tile; from then on the stores (and residual requests) of the iteration
+    // before and one k tile.
+    iteration(3, 0, 0, 0, PersistIter<true, true, IMM, NS, 0, false, false, true, true, PNLD + IMM>{});
+    iteration(4, 0, 0, 0, PersistIter<false, false, IMM + NS, NS, 1, false, false, true, true, PNLD + IMM + NS + NR>{});
     auto drain = [&](auto self, auto d) __attribute__((always_inline)) {
       constexpr int D = decltype(d)::value;
       if constexpr (D < DI) {
-        iteration(D + 3, 0, 0, 0, N{}, N{}, IC<IMM + D * NS>{}, IC<NS>{}, N{}, Y{}, Y{}, IC<PNLD + NS>{});
+        iteration(D + 3, 0, 0, 0, PersistIter<false, false, IMM + D * NS, NS, D, false, false, true, true, PNLD + NS + NR>{});
         self(self, IC<D + 1>{});
       }
     };
     drain(drain, IC<2>{});
-    iteration(DI + 3, 0, 0, 0, N{}, N{}, IC<0>{}, IC<0>{}, N{}, Y{}, Y{}, IC<PNLD + NS>{});
-    for (int kt = DI + 1; kt < nk - 3; ++kt) iteration(kt + 3, 0, 0, 0, N{}, N{}, IC<0>{}, IC<0>{}, N{}, Y{}, Y{}, IC<PNLD>{});
+    iteration(DI + 3, 0, 0, 0, PersistIter<false, false, 0, 0, 0, false, false, true, true, PNLD + NS>{});
+    for (int kt = DI + 1; kt < nk - 3; ++kt) iteration(kt + 3, 0, 0, 0, Plain{});
     tile_tail(ti);
   }
 
   // ---- the last tile's output ---------------------------------------------------------------------
+  if constexpr (RES) __builtin_amdgcn_s_waitcnt(0x0F70 | PNLD);  // the residual values requested in the last iteration
   convert_begin(conv_sc);
-  convert_half(0, conv_sc);
+  convert_half(0, conv_sc, false);
 #pragma unroll
   for (int s = 0; s < 16; ++s) store_piece(s);
-  convert_half(1, conv_sc);
+  if constexpr (RES) {
+    // the second half's residual values (only the first NS of them were requested ahead)
+    u32x2 res_late[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) res_late[r] = residual_piece(16 + r);
+    convert_half(1, conv_sc, false);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) add_residual(held[1][r], res_late[r]);
+  } else {
+    convert_half(1, conv_sc, false);
+  }
 #pragma unroll
   for (int s = 16; s < 32; ++s) store_piece(s);
   __builtin_amdgcn_s_waitcnt(0x0070);  // the unused loads of the last tail land before the LDS is given back
 }
 
-// workgroups of a persistent launch: two per CU, a multiple of the 8 XCDs
 static int persist_grid() {
   static const int grid = [] {
     int dev = 0, cus = 0;
@@ -362,9 +481,14 @@ static int persist_grid() {
 }
 
 bool gemm_i8_persist_covers(int epi, const GemmArgs& a) {
-  const int mode = knob_or(KNOB_GEMM_PERSIST, 0);
+  // 0: off; 1 (default): the scale + bias and GELU epilogues, where it measures faster than one
+  // workgroup per tile (qkv -20 %, lin1 -5 % at 65536 rows), from two tiles per workgroup on; 2: also the
+  // residual epilogue (measured 4-10 % slower than three workgroups per CU) and any tile count
+  const int mode = knob_or(KNOB_GEMM_PERSIST, 1);
   if (mode <= 0) return false;
-  if (epi != EPI_SCALE_BIAS_BF16 && epi != EPI_GELU_BF16) return false;
+  if (mode == 1 && epi == EPI_RESIDUAL_BF16) return false;
+  if (epi != EPI_SCALE_BIAS_BF16 && epi != EPI_GELU_BF16 && epi != EPI_RESIDUAL_BF16) return false;
+  if (epi == EPI_RESIDUAL_BF16 && a.ld_res >= (1ll << 23)) return false;
   if (a.M % PBM != 0 || a.N % PBN != 0 || a.K / GBK < 12) return false;
   if (a.dst_row || a.tile_counters || a.ldo >= (1ll << 23)) return false;  // 32-bit row offsets inside a tile
   // worth it from two tiles per workgroup on (mode 2: wherever it is built)
@@ -373,6 +497,8 @@ bool gemm_i8_persist_covers(int epi, const GemmArgs& a) {
 
 int gemm_i8_persist_launch(int epi, const GemmArgs& a0, hipStream_t stream) {
   GemmArgs a = a0;
+  // start delay of every second workgroup: knob x 64 cycles per k tile of a tile's K loop
+  a.skew = min(max(knob_or(KNOB_GEMM_PERSIST_SKEW, 22), 0) * (a.K / GBK), 1 << 16);
   a.tiles_m = a.M / PBM;
   a.tiles_n = a.N / PBN;
   a.group_m = a.tiles_n <= 6 ? 1 : 1024 / PBM;
@@ -387,6 +513,7 @@ int gemm_i8_persist_launch(int epi, const GemmArgs& a0, hipStream_t stream) {
     else hipLaunchKernelGGL((gemm_i8_persist_kernel<E, 8, 16, false>), dim3(grid), dim3(256), 0, stream, a);                      \
   } while (0)
   if (epi == EPI_GELU_BF16) SF_PERSIST(EPI_GELU_BF16);
+  else if (epi == EPI_RESIDUAL_BF16) SF_PERSIST(EPI_RESIDUAL_BF16);
   else SF_PERSIST(EPI_SCALE_BIAS_BF16);
 #undef SF_PERSIST
   return check_launch("gemm_i8_persist_kernel");

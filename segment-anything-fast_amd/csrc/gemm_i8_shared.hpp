@@ -22,6 +22,7 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int group_m;     // row tiles per scheduling group
   int stream_out;  // outputs without residual that exceed the 256 MB last-level cache
+  int skew;        // persistent kernel: start delay of the workgroups in odd wave slots, units of 64 cycles
   int row_pitch;            // bytes between consecutive rows of X / W: K (row-major) or 64 (K-block major)
   int64_t x_kstep, w_kstep; // bytes between consecutive 64-byte k tiles: 64, or rows * 64
   const unsigned short* residual;  // EPI_RESIDUAL: (rows, N) bf16, row stride ld_res

@@ -30,6 +30,7 @@ enum Knob {
   KNOB_GEMM_TILE,         // SAMFAST_GEMM_TILE: 64 / 128 forces the small / large tile of the three-per-CU kernel
   KNOB_GEMM_SMALL_BELOW,  // SAMFAST_GEMM_SMALL_BELOW: tile count below which the small tile is taken
   KNOB_GEMM_PERSIST,      // SAMFAST_GEMM_PERSIST: 0 off, 1 where it pays, 2 wherever it is built
+  KNOB_GEMM_PERSIST_SKEW, // SAMFAST_GEMM_PERSIST_SKEW: start delay of every second resident workgroup, 64 cycles per k tile
   KNOB_GEMM_SPLITK,       // SAMFAST_GEMM_SPLITK: 0 off, 1 where it pays (launches that leave the GPU half empty)
   KNOB_ATTN_WAVES,        // SAMFAST_ATTN_WAVES: 4 / 8 wavefronts per global-attention workgroup
   KNOB_COUNT

@@ -522,6 +522,10 @@ def test_gemm_two_and_three_workgroups_per_cu_agree(M, N, K, epi):
     (8320, 3072, 1024, "gelu"),
     (1024, 1280, 5120, "none"),    # fewer tiles than workgroups: one tile each, 80 k tiles
     (65536, 3840, 1280, "none"),   # the qkv Linear at full size: streaming stores, 15 tiles per workgroup
+    (32768, 1280, 1280, "residual"),          # proj: 1280 tiles, lists of 2 and 3
+    (32768, 1280, 5120, "residual_in_place"),  # lin2 as the block calls it: output buffer = residual buffer
+    (16384, 768, 3072, "residual"),           # ViT-B lin2
+    (24576, 1024, 1024, "residual_in_place"),  # ViT-L proj: 16 k tiles, stores over 8 iterations
 ])
 def test_gemm_persistent_form_agrees(M, N, K, epi):
     """The persistent form of the 128 x 256 kernel (resident workgroups that walk a list of tiles,
@@ -537,11 +541,23 @@ def test_gemm_persistent_form_agrees(M, N, K, epi):
     L = _lib.LAYOUT_KB64
     xq, sx = ops.quant_rowwise(x.cuda(), L)
     wq, sw = ops.quant_rowwise(w.cuda(), L)
-    code = {"none": _lib.EPILOGUE_NONE, "gelu": _lib.EPILOGUE_GELU}[epi]
-    want = ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L)
+    code = {"none": _lib.EPILOGUE_NONE, "gelu": _lib.EPILOGUE_GELU}.get(epi, _lib.EPILOGUE_RESIDUAL)
+    res = None
+    if code == _lib.EPILOGUE_RESIDUAL:
+        res = torch.randn((M, N), generator=g).to(torch.bfloat16).cuda()
+
+    def run():
+        if res is None:
+            return ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L)
+        if epi == "residual_in_place":
+            buf = res.clone()
+            return ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, residual=buf, out=buf, layout=L)
+        return ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, residual=res, layout=L)
+
+    want = run()
     with _lib.knobs(SAMFAST_GEMM_PERSIST=2):
-        got = ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L)
-        again = ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L)
+        got = run()
+        again = run()
     torch.cuda.synchronize()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     assert torch.equal(again.view(torch.int16), want.view(torch.int16))
@@ -553,6 +569,9 @@ def test_gemm_persistent_form_agrees(M, N, K, epi):
     ref = orq.scale_bias_epilogue(acc, sx_r, sw_r, bias.cpu())
     sample = got[rows.cuda()].cpu()
     if epi == "none":
+        assert torch.equal(sample.view(torch.int16), ref.view(torch.int16))
+    elif res is not None:
+        ref = (ref.float() + res[rows.cuda()].cpu().float()).to(torch.bfloat16)  # bf16 add of bf16 operands
         assert torch.equal(sample.view(torch.int16), ref.view(torch.int16))
     else:
         act = torch.nn.functional.gelu(ref.float()).to(torch.bfloat16).float()
