@@ -4,9 +4,13 @@
 `sam_model_registry[name](checkpoint=None)` builds the float model;
 `sam_model_fast_registry[name](checkpoint=None, compile_mode='max-autotune',
 dtype=torch.bfloat16)` returns it in eval mode and `dtype`.  The fast path here
-is the HIP kernels behind Attention / Int8DynamicLinear, so `compile_mode` is
-accepted for signature compatibility and not used: nothing is traced or
-autotuned.
+is the HIP kernels behind Attention / Int8DynamicLinear; nothing is traced or
+autotuned.  What `compile_mode` keeps of the reference's
+`torch.compile(sam.image_encoder, mode=compile_mode)` (:67-71) is the part that
+matters at small batch: with any mode but None the image encoder is wrapped in
+`graphs.ReplayedEncoder`, which records one forward per input shape into a HIP
+graph and replays it while the batch is launch-bound (up to four images).
+`compile_mode=None` leaves the encoder as it is.
 
 Only the image encoder is constructed (hyper-parameters from :14-44,102-120);
 checkpoint keys that belong to the prompt encoder / mask decoder are ignored on
@@ -79,8 +83,11 @@ def _apply_eval_dtype_sam(model: Sam, dtype):
 
 
 def _fast(builder, checkpoint, compile_mode, dtype):
-    del compile_mode  # no tracing compiler on this path
-    return _apply_eval_dtype_sam(builder(checkpoint), dtype)
+    sam = _apply_eval_dtype_sam(builder(checkpoint), dtype)
+    if compile_mode is not None:
+        from .graphs import ReplayedEncoder
+        sam.image_encoder = ReplayedEncoder(sam.image_encoder, compile_mode)
+    return sam
 
 
 def build_sam_fast_vit_h(checkpoint=None, compile_mode="max-autotune", dtype=torch.bfloat16):

@@ -115,6 +115,8 @@ def apply_fake_sparsity(model: nn.Module,
                         filter_fn: Optional[Callable[[nn.Module, str], bool]] = None) -> None:
     """Zero, in place, the 2 smallest-magnitude weights of every 4 of each selected
     nn.Linear (sparse.py:6-25).  Dense storage, dense kernels: accuracy simulation only."""
+    from .graphs import invalidate_recordings
+    invalidate_recordings(model)
     sel = _wrap(filter_fn)
     for name, mod in model.named_modules():
         if isinstance(mod, nn.Linear) and sel(mod, name):

@@ -21,6 +21,7 @@ def init_encoder_weights(encoder: torch.nn.Module, seed: int = 0) -> Dict[str, t
     """Fill `encoder` in place (fp32, CPU generator => identical on every machine);
     returns its state dict."""
     gen = torch.Generator(device="cpu").manual_seed(seed)
+    encoder = getattr(encoder, "_orig_mod", encoder)  # the fast registry's replay wrapper: same names as the bare encoder
     with torch.no_grad():
         for name, p in sorted(encoder.named_parameters(), key=lambda kv: kv[0]):
             t = torch.empty(p.shape, dtype=torch.float32)

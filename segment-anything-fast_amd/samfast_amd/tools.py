@@ -5,6 +5,9 @@ def replace_with_custom_fn_if_matches_filter(model, replacement_fn, filter_fn, c
     """Walk `model`; every child for which filter_fn(child, fully_qualified_name)
     holds is replaced by replacement_fn(child), other children are searched
     recursively.  (tools.py:1-19)"""
+    if cur_fqn == "":
+        from .graphs import invalidate_recordings
+        invalidate_recordings(model)  # recorded graphs hold the addresses of the modules replaced below
     for name, child in list(model.named_children()):
         fqn = name if cur_fqn == "" else f"{cur_fqn}.{name}"
         if filter_fn(child, fqn):

@@ -153,6 +153,32 @@ def test_registry_surface():
     assert sam.preprocess(img).shape == (1, 3, 1024, 1024)
 
 
+def test_fast_registry_wraps_the_encoder_for_graph_replay():
+    """compile_mode of the fast builders (build_sam.py:67-71 of the reference compiles the encoder
+    with it): any mode wraps the encoder for HIP-graph replay, None leaves it bare.  The wrapper
+    forwards attributes, keeps the reference's post-compile state-dict prefix and drops its
+    recordings whenever weights or modules are replaced."""
+    import samfast_amd
+    from samfast_amd import tools
+    from samfast_amd.graphs import ReplayedEncoder
+    from samfast_amd.modeling import ImageEncoderViT
+    sam = samfast_amd.sam_model_fast_registry["vit_b"]()
+    enc = sam.image_encoder
+    assert isinstance(enc, ReplayedEncoder) and enc.compile_mode == "max-autotune"
+    assert enc.img_size == 1024 and len(enc.blocks) == 12 and isinstance(enc._orig_mod, ImageEncoderViT)
+    assert all(k.startswith("_orig_mod.") for k in enc.state_dict())
+    bare = samfast_amd.sam_model_fast_registry["vit_b"](compile_mode=None).image_encoder
+    assert isinstance(bare, ImageEncoderViT)
+    assert not enc.replays(torch.zeros(1, 3, 1024, 1024))  # CPU tensors run eagerly
+    for mutate in (lambda: tools.replace_with_custom_fn_if_matches_filter(enc, lambda m: m, lambda m, f: False),
+                   lambda: enc.load_state_dict(enc.state_dict()),
+                   lambda: samfast_amd.apply_fake_sparsity(sam, lambda m, f: False),
+                   lambda: enc.float()):
+        enc._graphs["stale"] = object()
+        mutate()
+        assert not enc._graphs
+
+
 def test_module_signatures_follow_reference():
     from samfast_amd.modeling import Attention, Block, ImageEncoderViT, MLPBlock
     assert list(inspect.signature(Attention.__init__).parameters)[1:] == [

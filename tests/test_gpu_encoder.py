@@ -132,6 +132,50 @@ def test_predictor_set_torch_image():
     assert f.shape == (1, 256, 64, 64) and f.dtype == torch.bfloat16 and torch.isfinite(f.float()).all()
 
 
+def test_fast_registry_replays_a_graph_bit_equal_to_eager():
+    """The encoder the fast registry returns replays a HIP graph for small batches (what the
+    reference's compile_mode='max-autotune' gives, build_sam.py:67-71): bit-equal to the eager
+    forward, replay after replay, also on a second image; a module swap drops the recording;
+    a batch beyond the launch-bound range runs eagerly."""
+    import samfast_amd
+    from samfast_amd.graphs import ReplayedEncoder
+    from samfast_amd.sparse import mlp_only
+    from samfast_amd.synthetic import init_encoder_weights, make_images
+    sam = samfast_amd.sam_model_fast_registry["vit_b"]()
+    init_encoder_weights(sam.image_encoder, seed=0)
+    sam = sam.cuda()
+    samfast_amd.apply_dynamic_quant(sam.image_encoder)
+    enc = sam.image_encoder
+    assert isinstance(enc, ReplayedEncoder)
+    imgs = make_images(2, seed=3).to(torch.bfloat16).cuda()
+    a, b = imgs[:1], imgs[1:]
+    with torch.no_grad():
+        eager_a, eager_b = enc._orig_mod(a), enc._orig_mod(b)
+        assert enc.replays(a)
+        first, other, again = enc(a), enc(b), enc(a)
+        torch.cuda.synchronize()
+        assert len(enc._graphs) == 1
+        assert torch.equal(first, eager_a) and torch.equal(again, eager_a) and torch.equal(other, eager_b)
+        # the predictor goes through the same wrapper
+        pred = samfast_amd.SamPredictor(sam)
+        raw = torch.rand(1, 3, 1024, 1024, device="cuda") * 255
+        pred.set_torch_image(raw, (1024, 1024))
+        want = enc._orig_mod(sam.preprocess(raw).to(torch.bfloat16))
+        assert torch.equal(pred.get_image_embedding(), want)
+        # swapping modules drops the recordings; the next forward records the new modules
+        samfast_amd.apply_sparse(enc, mlp_only)
+        assert not enc._graphs
+        sparse_eager = enc._orig_mod(a)
+        assert torch.equal(enc(a), sparse_eager) and torch.equal(enc(a), sparse_eager)
+        assert not torch.equal(sparse_eager, eager_a)
+        # eight images are not launch-bound: eager path, nothing recorded
+        big = make_images(8, seed=4).to(torch.bfloat16).cuda()
+        assert not enc.replays(big)
+        n = len(enc._graphs)
+        assert torch.equal(enc(big)[:1], enc._orig_mod(big[:1]))
+        assert len(enc._graphs) == n
+
+
 def test_fused_block_equals_module_composition():
     """Block.forward as nine fused launches against the same block run module by module
     (LayerNorm, window partition, residual adds and GELU in PyTorch-ROCm), windowed and global."""
