@@ -70,6 +70,9 @@ def parse():
                         "configuration); every other Linear dense int8")
     p.add_argument("--graph", action="store_true",
                    help="replay the forward as one HIP graph (launch-bound shapes, e.g. vit_b batch 1)")
+    p.add_argument("--also-graph", action="store_true",
+                   help="besides the eager launches, time the forward replayed as a HIP graph and through "
+                        "sam_model_fast_registry (hip_graph_replay / fast_registry_replay objects)")
     p.add_argument("--calibration-copy", action="store_true",
                    help="also run one 1 GiB device-to-device copy (a known-size reference for "
                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -547,7 +550,7 @@ def main():
         args.model, args.batch, args.steps, args.warmup, sparse_mlp=args.sparse_mlp,
         bf16_linears=args.bf16_linears, graph=args.graph, gpu_baseline=not args.no_gpu_baseline,
         calibration_copy=args.calibration_copy, yardsticks=args.library_yardsticks,
-        compiled_baseline=not args.no_gpu_baseline and not args.no_compiled_baseline)
+        compiled_baseline=not args.no_gpu_baseline and not args.no_compiled_baseline, also_graph=args.also_graph)
 
     result = {
         "metric": ("images/s ViT-H encoder bs16 1024^2" if (args.model, args.batch) == ("vit_h", 16)
@@ -560,7 +563,8 @@ def main():
         "data": "synthetic (seeded uniform images, random-init weights)",
         "config": main_run["config"],
     }
-    for k in ("hip_graph", "output_finite", "roofline", "kernels", "gpu_baseline", "library_yardsticks"):
+    for k in ("hip_graph", "output_finite", "roofline", "kernels", "gpu_baseline", "library_yardsticks",
+              "hip_graph_replay", "fast_registry_replay"):
         if k in main_run:
             result[k] = main_run[k]
 

@@ -79,6 +79,12 @@ const char* samfast_last_error(void);
  * Supported: hd in {64, 80}; (gw == 64 and N % 128 == 0) or (gh <= 15 and
  *   gw <= 16 and N <= 208); dtype SAMFAST_BF16 or SAMFAST_F16 (q, k, v, out and the tables
  *   all of that type; accumulation, softmax and bias in fp32 either way).
+ * Range of the bias in the window kernels: the two factors <q, rel_pos row> travel through the
+ *   matrix cores as 16-bit values already divided by sm_scale, so they carry the element type's
+ *   resolution and, for SAMFAST_F16, must satisfy |<q, rel_pos row>| < 65504 * sm_scale (about
+ *   7300 at head_dim 80, where the reference's fp16 einsum itself overflows at 65504); padding
+ *   keys are masked with a score of -60000 / sm_scale, so real scores have to stay well above that.
+ *   The global kernels keep the factors in fp32 and have no such limit.
  */
 int samfast_attn_relpos_fwd(
     const void* q, const void* k, const void* v,

@@ -385,15 +385,21 @@ _tile_counters = {}
 
 
 def tile_counters(rows: int, device) -> torch.Tensor:
-    """The zeroed int32 workspace samfast_gemm_i8_fused_quant wants (one entry per 128 rows), one
-    buffer per (device, stream): every launch leaves it zero again, and launches on one stream
-    cannot overlap."""
-    key = (str(device), torch.cuda.current_stream().cuda_stream)
+    """The zeroed int32 workspace samfast_gemm_i8_fused_quant wants (one entry per 128 rows).
+    Outside graph capture: one buffer per (device, stream) - launches on one stream cannot overlap -
+    whose entries are cleared on the stream before every use (a fill kernel): a launch leaves them
+    zero again, but one that ended early (an error, a killed kernel) would not, and nothing else
+    would ever notice.  Under capture: a buffer of the recording's own (from the graph's memory
+    pool), so that two recorded graphs replayed on different streams never share counters."""
     need = -(-rows // 128)
+    if torch.cuda.is_current_stream_capturing():
+        return torch.zeros(max(need, 1), dtype=torch.int32, device=device)
+    key = (str(device), torch.cuda.current_stream().cuda_stream)
     buf = _tile_counters.get(key)
     if buf is None or buf.numel() < need:
-        buf = torch.zeros(max(need, 1024), dtype=torch.int32, device=device)
+        buf = torch.empty(max(need, 1024), dtype=torch.int32, device=device)
         _tile_counters[key] = buf
+    buf[:need].zero_()
     return buf
 
 

@@ -206,6 +206,26 @@ def test_rising_maximum_along_the_keys(gh, gw, hd, ramp):
     _check(out, ref, f"rising max {gh}x{gw}x{hd} ramp {ramp}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_window_kernel_with_large_bias_factors(dtype):
+    """Relative-position tables 25 times the usual size: the bias factors <q, rel_pos row> reach
+    +-20, the 16-bit operands that carry them (pre-divided by the softmax scale) about +-180 -
+    inside the range include/samfast.h documents for fp16 - and the bias decides the softmax.
+    fp16 keeps the bar of the other tests; bf16's eight-bit mantissa puts a factor of 20 on a grid
+    of 0.06, so its bar is widened by that much."""
+    from samfast_amd import ops
+    B, nH, gh, gw, hd = 3, 2, 14, 14, 80
+    q, k, v, rph, rpw = attn_inputs(B, nH, gh, gw, hd, seed=31, table_std=0.5, dtype=dtype)
+    ref = _oracle_tables(q, k, v, rph, rpw, (gh, gw))
+    out = ops.attn_relpos(q.cuda(), k.cuda(), v.cuda(), rph.cuda(), rpw.cuda(), (gh, gw))
+    torch.cuda.synchronize()
+    diff = (out.float().cpu() - ref.float()).abs()
+    print(f"large bias {dtype}: max-abs {diff.max().item():.3e} mean-abs {diff.mean().item():.3e}", flush=True)
+    assert torch.isfinite(out.float()).all()
+    loose = 1 if dtype == torch.float16 else 8
+    assert diff.max().item() <= loose * MAX_ABS and diff.mean().item() <= loose * MEAN_ABS
+
+
 @pytest.mark.parametrize("hd,gh", [(80, 64), (64, 64), (80, 8)])
 def test_global_kernel_wave_count_variants_agree(hd, gh):
     """The global kernel runs with 128 or 256 queries per workgroup (4 or 8 wavefronts); the choice

@@ -465,6 +465,60 @@ def test_gemm_with_output_quantiser_equals_separate_launches(M, N, K, kind):
         del y, q, s, y_ref, q_ref, s_ref, xq, wq, res
 
 
+@pytest.mark.parametrize("M,N,K,kind", [
+    (333, 5120, 1280, "gelu"),       # 20 column tiles, last row tile partial: quantiser inside the kernel
+    (333, 1280, 1280, "ln"),         # 5 column tiles, LayerNorm + quantiser inside the kernel
+    (333, 1280, 5120, "ln"),
+    (333, 1280, 1280, "residual"),   # residual + plain quantiser: two launches behind the same entry point
+    (200, 3072, 768, "gelu"), (200, 768, 3072, "ln"),
+])
+def test_gemm_with_output_quantiser_against_the_oracle(M, N, K, kind):
+    """samfast_gemm_i8_fused_quant against the CPU oracle directly (the other tests of this entry
+    point compare it with the separate launches, which share its device code).
+    y: the Linear (+ residual) bit for bit, GELU within one bf16 step.  Codes and scales: what the
+    oracle's row quantiser makes of the y the call returned, bit for bit; behind a LayerNorm the
+    oracle normalises y in fp32 (F.layer_norm) and rounds to bf16 first, and codes may differ by
+    one step where the two LayerNorms round a value differently."""
+    from samfast_amd import _lib, ops
+    print(f"case fused quant vs oracle M={M} N={N} K={K} {kind}", flush=True)
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16)
+    x[torch.randperm(M, generator=g)[:2]] *= 20.0
+    w = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    bias = torch.randn((N,), generator=g) * 0.02
+    res = torch.randn((M, N), generator=g).to(torch.bfloat16)
+    gamma = (1 + 0.1 * torch.randn(N, generator=g)).to(torch.bfloat16)
+    beta = (0.1 * torch.randn(N, generator=g)).to(torch.bfloat16)
+    L = _lib.LAYOUT_KB64
+    xq, sx = ops.quant_rowwise(x.cuda(), L)
+    wq, sw = ops.quant_rowwise(w.cuda(), L)
+    epilogue = _lib.EPILOGUE_GELU if kind == "gelu" else _lib.EPILOGUE_RESIDUAL
+    y, yq, sy = ops.gemm_i8_fused_quant(
+        xq, sx, wq, sw, bias.cuda(), epilogue, residual=res.cuda() if kind != "gelu" else None, layout=L,
+        ln=(gamma.cuda(), beta.cuda(), 1e-6) if kind == "ln" else None, out_layout=_lib.LAYOUT_ROWMAJOR)
+    torch.cuda.synchronize()
+    y, yq, sy = y.cpu(), yq.cpu().numpy(), sy.cpu().numpy()
+    lin = orq.dynamic_int8_linear(x, w, bias)  # bf16
+    if kind == "gelu":
+        want = torch.nn.functional.gelu(lin.float()).to(torch.bfloat16)
+        assert torch.allclose(y.float(), want.float(), rtol=2 ** -7, atol=1e-6)
+        assert (y == want).float().mean() >= 0.99
+    else:
+        want = (lin.float() + res.float()).to(torch.bfloat16)
+        assert torch.equal(y.view(torch.int16), want.view(torch.int16))
+    if kind == "ln":
+        normed = torch.nn.functional.layer_norm(y.float(), (N,), gamma.float(), beta.float(), 1e-6).to(torch.bfloat16)
+        q_ref, s_ref = orq.quantize_rows_absmax(normed)
+        assert np.allclose(sy, s_ref, rtol=2 ** -7)
+        steps = np.abs(yq.astype(np.int32) - q_ref.astype(np.int32))
+        # a value the two LayerNorms round differently moves its code by a step (its row's whole codes
+        # where that value is the row's absmax): nearly all codes agree, none is off by more than 2
+        assert steps.max() <= 2 and (steps == 0).mean() >= 0.97, (int(steps.max()), float((steps == 0).mean()))
+    else:
+        q_ref, s_ref = orq.quantize_rows_absmax(y)
+        assert np.array_equal(sy, s_ref) and np.array_equal(yq, q_ref)
+
+
 def test_gemm_with_output_quantiser_in_place_residual():
     """lin2's form: the output overwrites the residual stream it reads (out = residual)."""
     from samfast_amd import _lib, ops

@@ -162,6 +162,40 @@ def test_apply_sparse_mlp_only_module_and_encoder():
     assert torch.isfinite(out).all() and cos >= 0.999, cos
 
 
+def test_apply_sparse_every_linear_as_the_reference_does():
+    """apply_sparse(model) with no filter - the reference's own scope (sparse.py:28-32 swaps every
+    Linear): qkv, proj, lin1 and lin2 of a windowed and a global ViT-H block all become 2:4-sparse
+    int8 Linears (proj without its row scatter, so windowed blocks take the module-by-module route
+    or the in-place window kernel), and the encoder output follows the oracle that prunes and
+    quantises all four the same way."""
+    from functools import partial
+    from samfast_amd import apply_sparse
+    from samfast_amd.modeling import ImageEncoderViT
+    from samfast_amd.sparse import Int8Sparse24Linear
+    from samfast_amd.synthetic import init_encoder_weights, make_images
+    from oracle import image_encoder as oe
+
+    cfg = oe.EncoderConfig(embed_dim=1280, depth=2, num_heads=16, global_attn_indexes=(1,))
+    enc = ImageEncoderViT(depth=2, embed_dim=1280, num_heads=16, global_attn_indexes=(1,),
+                          window_size=14, use_rel_pos=True, mlp_ratio=4,
+                          norm_layer=partial(torch.nn.LayerNorm, eps=1e-6))
+    sd = {k: v.clone() for k, v in init_encoder_weights(enc, seed=7).items()}
+    enc = enc.eval().to(torch.bfloat16).cuda()
+    apply_sparse(enc)
+    for blk in enc.blocks:
+        for lin in (blk.attn.qkv, blk.attn.proj, blk.mlp.lin1, blk.mlp.lin2):
+            assert isinstance(lin, Int8Sparse24Linear)
+    x = make_images(1, seed=6).to(torch.bfloat16)
+    sparse = lambda a, w, b: orq.sparse24_int8_linear(a, w, b).float()
+    with torch.no_grad():
+        out = enc(x.cuda()).float().cpu()
+        sd_r = {k: v.to(torch.bfloat16).float() for k, v in sd.items()}
+        ref = oe.encoder_forward(sd_r, x.float(), cfg, linear=sparse, use_sdpa=True)
+    cos = torch.nn.functional.cosine_similarity(out.flatten(1), ref.flatten(1), dim=1).min().item()
+    print(f"all-Linears sparse slice: cosine {cos:.6f}", flush=True)
+    assert torch.isfinite(out).all() and cos >= 0.999, cos
+
+
 def test_seeded_sweep_of_ragged_shapes_sparse_bit_exact():
     """Twenty random shapes: the 2:4 GEMM's accumulators equal the dense product with the pruned
     int8 matrix bit for bit (K in steps of 128 from 256, as the sparse kernel requires)."""
