@@ -42,15 +42,16 @@ class record_launches:
         """{kernel: dict(launches, work, unit, ms)} after synchronising."""
         torch.cuda.synchronize()
         out = {}
-        for name, work, unit, e0, e1 in self.entries:
-            d = out.setdefault(name, dict(launches=0, work=0.0, unit=unit, ms=0.0))
+        for name, work, unit, e0, e1, nbytes in self.entries:
+            d = out.setdefault(name, dict(launches=0, work=0.0, unit=unit, ms=0.0, bytes=0.0))
             d["launches"] += 1
             d["work"] += work
+            d["bytes"] += nbytes
             d["ms"] += e0.elapsed_time(e1)
         return out
 
 
-def _timed(name: str, work: float, unit: str, launch):
+def _timed(name: str, work: float, unit: str, launch, nbytes: float = 0.0):
     log = _launch_log
     if log is None:
         return launch()
@@ -59,7 +60,7 @@ def _timed(name: str, work: float, unit: str, launch):
     e0.record()
     code = launch()
     e1.record()
-    log.append((name, work, unit, e0, e1))
+    log.append((name, work, unit, e0, e1, nbytes))
     return code
 
 
@@ -139,7 +140,8 @@ def attn_relpos(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
             q.data_ptr(), k.data_ptr(), v.data_ptr(), rel_pos_h.data_ptr(), rel_pos_w.data_ptr(),
             out.data_ptr(), B, nH, gh, gw, hd,
             *_bnhd_strides(q), *_bnhd_strides(k), *_bnhd_strides(v), *_bnhd_strides(out),
-            _dtype_code(q), scale, _stream()))
+            _dtype_code(q), scale, _stream()),
+        nbytes=0.0 if gw == 64 else 4.0 * B * nH * N * hd * q.element_size())
     _lib.check(code, "attn_relpos_fwd")
     return out
 
@@ -175,7 +177,8 @@ def attn_relpos_windowed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
             rel_pos_w.data_ptr(), pad_k.data_ptr(), pad_v.data_ptr(), out.data_ptr(),
             B, nH, H, W, window, hd,
             *_bnhd_strides(q), *_bnhd_strides(k), *_bnhd_strides(v), *_bnhd_strides(o),
-            _dtype_code(q), float(scale), _stream()))
+            _dtype_code(q), float(scale), _stream()),
+        nbytes=4.0 * nwin * nH * nt * hd * q.element_size())
     _lib.check(code, "attn_relpos_windowed_fwd")
     return out
 
