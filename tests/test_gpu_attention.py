@@ -226,6 +226,29 @@ def test_window_kernel_with_large_bias_factors(dtype):
     assert diff.max().item() <= loose * MAX_ABS and diff.mean().item() <= loose * MEAN_ABS
 
 
+@pytest.mark.parametrize("B,nH,gh,gw,hd", [(5, 3, 14, 14, 80), (3, 2, 14, 14, 64), (2, 2, 7, 9, 80),
+                                            (2, 2, 13, 16, 64), (2, 2, 5, 3, 80), (2, 2, 15, 13, 80)])
+def test_both_window_key_layouts_vs_oracle(B, nH, gh, gw, hd):
+    """The window kernel exists with the keys in token order (attn_window_kernel) and as grid rows
+    padded to 16 (attn_window_rows_kernel, SAMFAST_ATTN_WINDOW_ROWS=1, built for gh <= 14).  Each is held to the
+    oracle's bar on its own, with the tables and with caller-computed bias factors; a window of 15
+    rows only fits the first."""
+    from samfast_amd import _lib, ops
+    print(f"case window layouts B={B} nH={nH} grid={gh}x{gw} hd={hd}", flush=True)
+    q, k, v, rph, rpw = attn_inputs(B, nH, gh, gw, hd, seed=17)
+    ref = _oracle_tables(q, k, v, rph, rpw, (gh, gw))
+    qb, kb, vb, rel_h, rel_w = bias_inputs(B, nH, gh, gw, hd, seed=18)
+    ref_b = ora.attention_rel_h_rel_w(qb, kb, vb, rel_h, rel_w, compute_dtype=torch.float32)
+    for rows in (0, 1):
+        with _lib.knobs(SAMFAST_ATTN_WINDOW_ROWS=rows):
+            out = ops.attn_relpos(q.cuda(), k.cuda(), v.cuda(), rph.cuda(), rpw.cuda(), (gh, gw))
+            out_b = ops.attn_relpos_bias(qb.cuda(), kb.cuda(), vb.cuda(), rel_h.cuda().squeeze(-1),
+                                         rel_w.cuda().squeeze(-2))
+            torch.cuda.synchronize()
+        _check(out, ref, f"tables, rows layout {rows}")
+        _check(out_b, ref_b, f"bias factors, rows layout {rows}")
+
+
 @pytest.mark.parametrize("hd,gh", [(80, 64), (64, 64), (80, 8)])
 def test_global_kernel_wave_count_variants_agree(hd, gh):
     """The global kernel runs with 128 or 256 queries per workgroup (4 or 8 wavefronts); the choice
