@@ -626,8 +626,14 @@ __global__ __launch_bounds__(256, (TM == 4 ? 1 : 2)) void gemm_i8_kernel(GemmArg
 // (each wave 32 x 64: 1 x 2 tiles, 32 accumulators, 27 KB of LDS) for launches whose large tiles
 // would leave most of the GPU's workgroup slots empty (4096 rows of a single image): four times
 // the workgroups, each a quarter of the work.
+// KSPLIT = 2 (64 x 128 tiles only) puts eight wavefronts on a tile: wavefronts 0-3 take the even k
+// tiles, wavefronts 4-7 the odd ones, each half with operand stages of its own, so the chain of
+// dependent iterations a single small launch has to sit through is half as long (a 4096-row lin2 at
+// K = 3072 is 384 workgroups of 48 iterations: one round, latency-bound).  The two partial sums are
+// int32 and meet in LDS after the loop - integer addition is order-free, so the result has the
+// same bits - and wavefronts 0-3 run the epilogue.
 // =============================================================================================
-template <int BM, int BN>
+template <int BM, int BN, int KSPLIT = 1>
 struct Gemm3Cfg {
   static constexpr int TMW = BM / 64, TNW = BN / 64;  // MFMA tiles per wavefront: rows, columns
   static constexpr int NST = 2;
@@ -636,26 +642,32 @@ struct Gemm3Cfg {
   static constexpr int EP_PITCH = BN * 2 + 32;        // staged output tile: row pitch in bytes
   static constexpr int SX_OFF = 0, SW_OFF = BM * 4, BIAS_OFF = SW_OFF + BN * 4, MAP_OFF = BIAS_OFF + BN * 4;
   static constexpr int SC_BYTES = MAP_OFF + BM * 4;
-  static constexpr int LDS_BYTES = NST * GSTAGE + SC_BYTES;
+  static constexpr int LDS_BYTES = KSPLIT * NST * GSTAGE + SC_BYTES;
+  static constexpr int THREADS = 256 * KSPLIT;
   static constexpr int CHUNKS = BN / 8;               // 16-byte pieces per output row
   static constexpr int ROWS_PER_PASS = 256 / CHUNKS;  // output rows the workgroup stores per pass
   static constexpr int PASSES = 64 / ROWS_PER_PASS;   // passes over a staged 64-row tile
-  static constexpr int MIN_WG = BM == 128 ? 3 : 4;
+  static constexpr int MIN_WG = BM == 128 ? 3 : (KSPLIT == 2 ? 2 : 4);
   static_assert(64 * EP_PITCH <= NST * GSTAGE, "a 64-row output tile must fit in the operand stages");
   static_assert((BM == 128 && BN == 256) || (BM == 64 && BN == 128), "tile shapes built");
+  static_assert(KSPLIT == 1 || (KSPLIT == 2 && BM == 64), "the K split is built for the small tile");
+  static_assert(KSPLIT == 1 || BM * BN * 4 <= KSPLIT * NST * GSTAGE, "the partial sums must fit in the operand stages");
 };
 
-template <int EPI, int BM, int BN>
-__global__ __launch_bounds__(256, (Gemm3Cfg<BM, BN>::MIN_WG)) void gemm_i8_kernel3(GemmArgs a) {
+template <int EPI, int BM, int BN, int KSPLIT = 1>
+__global__ __launch_bounds__((Gemm3Cfg<BM, BN, KSPLIT>::THREADS), (Gemm3Cfg<BM, BN, KSPLIT>::MIN_WG)) void gemm_i8_kernel3(GemmArgs a) {
   static_assert(EPI != EPI_I32, "bf16 epilogues only");
-  using C = Gemm3Cfg<BM, BN>;
+  using C = Gemm3Cfg<BM, BN, KSPLIT>;
   constexpr int TMW = C::TMW, TNW = C::TNW, NLD = C::NLD, GSTAGE = C::GSTAGE;
-  __shared__ __attribute__((aligned(16))) unsigned char lds[C::LDS_BYTES];
-  unsigned char* sc = lds + C::NST * GSTAGE;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_all[C::LDS_BYTES];
+  unsigned char* sc = lds_all + KSPLIT * C::NST * GSTAGE;
 
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x & 255;  // index inside the wavefront group (KSPLIT = 1: the workgroup)
   const int lane = tid & 63;
-  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave_u = wave_all & 3;    // wavefront inside its group of four
+  const int grp = wave_all >> 2;      // K split: which k tiles this group takes
+  unsigned char* lds = lds_all + grp * (C::NST * GSTAGE);  // the group's operand stages (and, group 0, the epilogue's tile)
   const int wm = wave_u >> 1, wn = wave_u & 1;
   const int lr = lane & 31, lh = lane >> 5;
 
@@ -730,15 +742,15 @@ __global__ __launch_bounds__(256, (Gemm3Cfg<BM, BN>::MIN_WG)) void gemm_i8_kerne
   const int b_off = BM * GLD + (wn * (BN / 2) + lr) * GLD + frag_chunk;
 
   const int nk = a.K / GBK;
-  dma_issue(0, 0);
-  for (int kt = 0; kt < nk; ++kt) {
-    const int stage_off = (kt & 1) * GSTAGE;
+  dma_issue(grp, 0);
+  for (int kt = grp, it = 0; kt < nk; kt += KSPLIT, ++it) {  // (K split: nk % KSPLIT == 0, both groups iterate alike)
+    const int stage_off = (it & 1) * GSTAGE;
     // own share of tile kt has landed; after the barrier the whole tile is visible and every
     // wavefront has left tile kt-1, whose stage may be refilled
     __builtin_amdgcn_s_waitcnt(0x0070);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    if (kt + 1 < nk) dma_issue(kt + 1, stage_off ^ GSTAGE);
+    if (kt + KSPLIT < nk) dma_issue(kt + KSPLIT, stage_off ^ GSTAGE);
     const unsigned char* src = lds + stage_off;
 #pragma unroll
     for (int step = 0; step < 2; ++step) {
@@ -754,6 +766,34 @@ __global__ __launch_bounds__(256, (Gemm3Cfg<BM, BN>::MIN_WG)) void gemm_i8_kerne
         for (int i = 0; i < TMW; ++i)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], acc[i][j], 0, 0, 0);
     }
+  }
+
+  bool active = true;  // whether this wavefront takes part in the epilogue's data movement
+  if constexpr (KSPLIT == 2) {
+    // the odd group's partial sums meet the even group's in LDS (the operand stages are free once
+    // every wavefront has left the loop); conflict-free: consecutive lanes, consecutive words
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    int* red = reinterpret_cast<int*>(lds_all);
+    if (grp == 1) {
+#pragma unroll
+      for (int i = 0; i < TMW; ++i)
+#pragma unroll
+        for (int j = 0; j < TNW; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) red[((wave_u * TMW * TNW + i * TNW + j) * 16 + r) * 64 + lane] = acc[i][j][r];
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    if (grp == 0) {
+#pragma unroll
+      for (int i = 0; i < TMW; ++i)
+#pragma unroll
+        for (int j = 0; j < TNW; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][j][r] += red[((wave_u * TMW * TNW + i * TNW + j) * 16 + r) * 64 + lane];
+    }
+    active = grp == 0;
   }
 
   // ---- epilogue, 64 rows at a time: pass h holds MFMA row tile h of both wavefront rows ----
@@ -778,7 +818,7 @@ __global__ __launch_bounds__(256, (Gemm3Cfg<BM, BN>::MIN_WG)) void gemm_i8_kerne
         if (a.bias) bvv[j] = *reinterpret_cast<const float*>(sc + C::BIAS_OFF + (wn * (BN / 2) + TNW * lr + j) * 4);
       }
     }
-    {
+    if (active) {
       unsigned char* dst = lds + (wm * 32 + 4 * lh) * C::EP_PITCH + (wn * (BN / 2) + TNW * lr) * 2;
       f32x4 sxv[4];
 #pragma unroll
@@ -828,7 +868,9 @@ __global__ __launch_bounds__(256, (Gemm3Cfg<BM, BN>::MIN_WG)) void gemm_i8_kerne
       const int t = C::ROWS_PER_PASS * p + rsub;
       return (t >> 5) * (BM / 2) + h * 32 + (t & 31);
     };
-    if (full) {
+    if (!active) {
+      // (the odd group only keeps the barrier count)
+    } else if (full) {
       u32x4 res[C::PASSES], val[C::PASSES];
       if (EPI == EPI_RESIDUAL_BF16) {
 #pragma unroll
@@ -961,17 +1003,22 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
     // 64 x 128 tiles when 128 x 256 ones would leave more than half of the 768 workgroup slots of
     // the GPU empty (SAMFAST_GEMM_TILE=64 / 128 forces either)
     const int ft = knob(KNOB_GEMM_TILE);
-    const bool small = ft != kKnobUnset ? ft == 64 : total < knob_or(KNOB_GEMM_SMALL_BELOW, 384);
+    const bool small = ft != kKnobUnset ? ft == 64 : total < knob_or(KNOB_GEMM_SMALL_BELOW, 385);
     if (small) {
       a.tiles_m = (int)((M + 63) / 64);
       a.tiles_n = (N + 127) / 128;
       a.group_m = a.tiles_n <= 6 ? 1 : 1024 / 64;
     }
     const int64_t total3 = (int64_t)a.tiles_m * a.tiles_n;
+    // small tiles that do not even fill the GPU's slots once, on a long K loop: two wavefront groups
+    // per tile, each on every second k tile (SAMFAST_GEMM_SPLITK=0 off, 2 wherever it is built)
+    const int sk = knob_or(KNOB_GEMM_SPLITK, 1);
+    const bool ksplit = small && (K / GBK) % 2 == 0 && (sk >= 2 || (sk == 1 && total3 <= 768 && K / GBK >= 12));
     const unsigned int grid3 = (unsigned int)(((total3 + 7) / 8) * 8);
 #define SF_GEMM3(E)                                                                                          \
   do {                                                                                                       \
-    if (small) hipLaunchKernelGGL((gemm_i8_kernel3<E, 64, 128>), dim3(grid3), dim3(256), 0, stream, a);      \
+    if (small && ksplit) hipLaunchKernelGGL((gemm_i8_kernel3<E, 64, 128, 2>), dim3(grid3), dim3(512), 0, stream, a); \
+    else if (small) hipLaunchKernelGGL((gemm_i8_kernel3<E, 64, 128>), dim3(grid3), dim3(256), 0, stream, a); \
     else hipLaunchKernelGGL((gemm_i8_kernel3<E, 128, 256>), dim3(grid3), dim3(256), 0, stream, a);           \
   } while (0)
     switch (epi) {

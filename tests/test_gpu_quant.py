@@ -534,7 +534,8 @@ def test_gemm_with_output_quantiser_in_place_residual():
 
 
 @pytest.mark.parametrize("M,N,K,epi", [(300, 1280, 1280, "residual"), (1000, 3840, 1280, "none"),
-                                       (513, 5120, 1280, "gelu"), (260, 1280, 5120, "residual_scatter")])
+                                       (513, 5120, 1280, "gelu"), (260, 1280, 5120, "residual_scatter"),
+                                       (4096, 768, 3072, "residual"), (4096, 2304, 768, "none")])
 def test_gemm_two_and_three_workgroups_per_cu_agree(M, N, K, epi):
     """The main GEMM kernel exists in three forms - three workgroups per CU with 128 x 256 tiles
     (single-buffered fragments, two LDS stages, epilogue staged 64 rows at a time; the default), the
@@ -560,13 +561,14 @@ def test_gemm_two_and_three_workgroups_per_cu_agree(M, N, K, epi):
             kw["dst_row"] = perm.cuda()
     outs = []
     # three per CU with 128 x 256 tiles, three (or more) per CU with 64 x 128 tiles, two per CU
-    for wg3, tile in ((1, 128), (1, 64), (0, 128)):
-        with _lib.knobs(SAMFAST_GEMM_WG3=wg3, SAMFAST_GEMM_TILE=tile):
+    # (the last: 64 x 128 tiles with the K loop split between two wavefront groups)
+    for wg3, tile, splitk in ((1, 128, 0), (1, 64, 0), (0, 128, 0), (1, 64, 2)):
+        with _lib.knobs(SAMFAST_GEMM_WG3=wg3, SAMFAST_GEMM_TILE=tile, SAMFAST_GEMM_SPLITK=splitk, SAMFAST_GEMM_PERSIST=0):
             out = torch.zeros_like(kw["residual"]) if "residual" in kw else None
             outs.append(ops.gemm_i8_fused(xq, sx, wq, sw, bias, code, layout=L, out=out, **kw).clone())
     torch.cuda.synchronize()
-    assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
-    assert torch.equal(outs[1].view(torch.int16), outs[2].view(torch.int16))
+    for i in (0, 1, 3):
+        assert torch.equal(outs[i].view(torch.int16), outs[2].view(torch.int16)), i
 
 
 @pytest.mark.parametrize("M,N,K,epi", [
@@ -649,8 +651,8 @@ def test_gelu_epilogue_all_bf16_inputs():
         sx = torch.ones((M,), dtype=torch.float32).cuda()
         wq = torch.zeros((N, K), dtype=torch.int8).cuda()
         sw = torch.ones((N,), dtype=torch.float32).cuda()
-        for name, wg3, tile in (("large", 1, 128), ("small", 1, 64), ("two", 0, 128)):
-            with _lib.knobs(SAMFAST_GEMM_WG3=wg3, SAMFAST_GEMM_TILE=tile):
+        for name, wg3, tile, splitk in (("large", 1, 128, 0), ("small", 1, 64, 0), ("two", 0, 128, 0), ("split", 1, 64, 2)):
+            with _lib.knobs(SAMFAST_GEMM_WG3=wg3, SAMFAST_GEMM_TILE=tile, SAMFAST_GEMM_SPLITK=splitk):
                 y = ops.gemm_i8_fused(xq, sx, wq, sw, bias, _lib.EPILOGUE_GELU)
                 torch.cuda.synchronize()
             assert torch.equal(y[0].view(torch.int16), y[M - 1].view(torch.int16))
