@@ -30,7 +30,7 @@
 // 16 consecutive output channels: slot (tile ta, MFMA row 8g + 4h + e) of a wave's 128 rows
 // holds W row 32g + 16*(ta/2) + 8h + 4*(ta%2) + e; the lane then writes 8 adjacent bf16 per
 // 16-byte store.
-#include "samfast_internal.hpp"
+#include "gemm_i8_sparse24_shared.hpp"
 #include <type_traits>
 
 // every fp32 step below is rounded on its own (no fused multiply-add), so results
@@ -39,45 +39,7 @@
 
 namespace samfast {
 
-typedef int i32x8 __attribute__((ext_vector_type(8)));
-
-constexpr int SBW = 256;  // W rows per workgroup (sparse operand = MFMA rows)
-constexpr int SBX = 128;  // X rows per workgroup (dense operand = MFMA columns)
-constexpr int SBK = 64;   // dense k per tile = one sparse MFMA k-step
-constexpr int S_OFF_W = SBX * SBK;             // X tile: 128 rows x 64 B
-constexpr int S_OFF_I = S_OFF_W + SBW * 32;    // Wc tile: 256 rows x 32 B
-constexpr int S_STAGE = S_OFF_I + SBW * 8;     // index tile: 256 rows x 8 B
 constexpr int S_NST = 4;                       // LDS stages (73 728 B: two workgroups per CU)
-
-enum { SEPI_I32 = 0, SEPI_SCALE_BIAS = 1, SEPI_GELU = 2, SEPI_RESIDUAL = 3 };
-
-struct SparseArgs {
-  const int8_t* x;
-  const int8_t* wc;
-  const int32_t* widx;
-  void* out;
-  const float* sx;
-  const float* sw;
-  const float* bias;
-  int64_t ldo;
-  int M, N, K;
-  int tiles_x, tiles_w;
-  int x_row_pitch;   // bytes between consecutive X rows: K (row-major) or 64 (K-block major)
-  int64_t x_kstep;   // bytes between consecutive 64-byte k tiles of X: 64, or M * 64
-  const unsigned short* residual;
-  int64_t ld_res;
-};
-
-// X rows: 64 B, four 16-byte chunks XOR-swizzled (same function as the dense kernel)
-SF_DEVICE int sp_swizzle_x(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
-// Wc rows: 32 B, two chunks; 8 / 16 consecutive rows read one chunk each without bank conflicts
-SF_DEVICE int sp_swizzle_w(int row) { return ((row >> 2) ^ (row >> 3)) & 1; }
-// LDS slot (0..255) of the W tile -> W row of the tile held there
-SF_DEVICE int sp_slot_to_row(int slot) {
-  const int ta = (slot >> 5) & 3, i = slot & 31;
-  const int g = i >> 3, h = (i >> 2) & 1, e = i & 3;
-  return (slot & 128) + 32 * g + 16 * (ta >> 1) + 8 * h + 4 * (ta & 1) + e;
-}
 
 template <int EPI>
 SF_DEVICE void sp24_epilogue(const SparseArgs& a, i32x16 (&acc)[4][2], int x0, int w0, int wa,
@@ -168,7 +130,6 @@ SF_DEVICE void sp24_epilogue(const SparseArgs& a, i32x16 (&acc)[4][2], int x0, i
 // stages; phase 2 walks it 8 rows at a time with 16 bytes per lane, so every store and
 // residual load instruction covers two whole 512-byte row segments.
 constexpr int SEP_STRIDE = 544;                     // tile row pitch in bytes
-constexpr int SEP_SCALE_BYTES = 512 + 1024 + 1024;  // sx[128], sw[256], bias[256] as fp32
 
 template <int EPI>
 SF_DEVICE void sp24_epilogue_staged(const SparseArgs& a, i32x16 (&acc)[4][2], unsigned char* lds,
@@ -533,6 +494,7 @@ static int sparse_common(int epi, const int8_t* xq, const float* sx, const int8_
   a.tiles_w = (N + SBW - 1) / SBW;
   const int64_t total = (int64_t)a.tiles_x * a.tiles_w;
   SF_REQUIRE(total < (1ll << 30), "gemm_i8_sparse24: too many tiles");
+  if (gemm_i8_sp24_persist_covers(epi, a)) return gemm_i8_sp24_persist_launch(epi, a, stream);
   const unsigned int grid = (unsigned int)(((total + 7) / 8) * 8);
   switch (epi) {
     case SEPI_I32:

@@ -34,6 +34,7 @@ enum Knob {
   KNOB_GEMM_SPLITK,       // SAMFAST_GEMM_SPLITK: 0 off, 1 where it pays (launches that leave the GPU half empty)
   KNOB_ATTN_WAVES,        // SAMFAST_ATTN_WAVES: 4 / 8 wavefronts per global-attention workgroup
   KNOB_ATTN_WINDOW_ROWS,  // SAMFAST_ATTN_WINDOW_ROWS: 1 = window keys as grid rows padded to 16 (attn_window_rows_kernel) where built
+  KNOB_SPARSE_PERSIST,    // SAMFAST_SPARSE_PERSIST: 2:4 GEMM, 0 = one workgroup per tile (default), 1 = resident workgroups from two tiles each on, 2 wherever built
   KNOB_COUNT
 };
 constexpr int kKnobUnset = INT32_MIN;
@@ -88,11 +89,13 @@ SF_DEVICE float xor32(float v) { return __shfl_xor(v, 32, 64); }
 // P = degree-7 least-squares fit (Chebyshev nodes) of log2 Phi(-z) on [0, 6]: |P - log2 Phi|
 // < 7e-6, i.e. h to 5e-6 relative in fp32 Horner form - a result that differs from the
 // correctly rounded bf16 value in about one of a thousand cases, by one step.  Beyond |x| = 6
-// h is held at Phi(-6) = 1e-9.  One transcendental and ten other instructions per value.
+// h is held at Phi(-6) = 1e-9.  One transcendental and ten other instructions per value: the two
+// clamps are median-of-three instructions (|x| as a source modifier), which unlike fminf / fmaxf
+// need no separate instruction to quiet a signalling NaN first.
 SF_DEVICE float gelu_erf(float x) {
 #pragma clang fp contract(fast)  // an approximation anyway: let the polynomial use FMAs
   const float ax = fabsf(x);
-  const float z = fminf(ax, 6.0f);
+  const float z = __builtin_amdgcn_fmed3f(ax, 0.0f, 6.0f);
   float p = -1.88962623e-06f;
   p = fmaf(p, z, 6.26814010e-05f);
   p = fmaf(p, z, -9.38867933e-04f);
@@ -102,7 +105,7 @@ SF_DEVICE float gelu_erf(float x) {
   p = fmaf(p, z, -1.15126915e+00f);
   p = fmaf(p, z, -9.99994340e-01f);
   const float h = __builtin_amdgcn_exp2f(p);
-  return fmaf(-ax, h, fmaxf(x, 0.f));
+  return fmaf(-ax, h, __builtin_amdgcn_fmed3f(x, 0.0f, 3.4028234664e38f));
 }
 
 // Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its

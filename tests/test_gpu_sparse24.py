@@ -96,6 +96,57 @@ def test_sparse24_fused_epilogues_equal_dense_kernels(M, N, K):
     assert torch.equal(buf.view(torch.int16), dense.view(torch.int16))
 
 
+@pytest.mark.parametrize("M,N,K,layout", [
+    (128, 256, 512, "rows"),        # one tile, the shortest K loop the resident form takes
+    (384, 512, 640, "rows"),        # six tiles, fewer tiles than workgroup slots
+    (1024, 768, 1280, "kb64"),      # K-block major codes as the encoder passes them
+    (66560, 1280, 1280, "kb64"),    # 2600 tiles: five per resident workgroup, uneven lists
+    (8192, 5120, 1280, "kb64"),     # lin1 shape: 1280 tiles
+    (4096, 1280, 5120, "kb64"),     # lin2 shape: 160 tiles, 80 k-steps
+])
+def test_sparse24_resident_form_agrees(M, N, K, layout):
+    """The resident-workgroup form of the 2:4 kernel (tile lists, the previous tile's output produced
+    at the top of the next tile) against the one-workgroup-per-tile form, bit for bit over the whole
+    output and for every epilogue (scale + bias, GELU, residual, residual in place), and against the
+    dense kernel on the pruned weight."""
+    from samfast_amd import _lib, ops
+    print(f"case sparse resident M={M} N={N} K={K} {layout}", flush=True)
+    g = torch.Generator().manual_seed(M + N + K)
+    xq = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).cuda()
+    wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    sx = (torch.rand(M, generator=g) * 1e-2 + 1e-3).cuda()
+    sw = (torch.rand(N, generator=g) * 1e-3 + 1e-4).cuda()
+    bias = (torch.randn(N, generator=g) * 0.1).cuda()
+    res = torch.randn((M, N), generator=g).to(torch.bfloat16).cuda()
+    wd = torch.from_numpy(_pruned_int8(wq)).cuda()
+    wc, widx = ops.prune24_pack(wq.cuda())
+    L = _lib.LAYOUT_ROWMAJOR
+    if layout == "kb64":
+        L = _lib.LAYOUT_KB64
+        xq, wd = ops.to_kb64(xq), ops.to_kb64(wd)
+
+    def run(epi, in_place=False):
+        if epi != _lib.EPILOGUE_RESIDUAL:
+            return ops.gemm_i8_sparse24_fused(xq, sx, wc, widx, sw, bias, epi, layout=L)
+        if in_place:
+            buf = res.clone()
+            return ops.gemm_i8_sparse24_fused(xq, sx, wc, widx, sw, bias, epi, residual=buf, out=buf, layout=L)
+        return ops.gemm_i8_sparse24_fused(xq, sx, wc, widx, sw, bias, epi, residual=res, layout=L)
+
+    for epi in (_lib.EPILOGUE_NONE, _lib.EPILOGUE_GELU, _lib.EPILOGUE_RESIDUAL):
+        with _lib.knobs(SAMFAST_SPARSE_PERSIST=0):
+            want = run(epi)
+        with _lib.knobs(SAMFAST_SPARSE_PERSIST=2):
+            got = run(epi)
+            again = run(epi, in_place=True)
+        kw = {"residual": res} if epi == _lib.EPILOGUE_RESIDUAL else {}
+        dense = ops.gemm_i8_fused(xq, sx, wd, sw, bias, epi, layout=L, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), epi
+        assert torch.equal(again.view(torch.int16), want.view(torch.int16)), epi
+        assert torch.equal(dense.view(torch.int16), want.view(torch.int16)), epi
+
+
 def test_sparse24_full_size_equals_dense_kernel():
     """lin1 of ViT-H at batch 16 (65536 x 5120 x 1280): accumulators of the sparse kernel
     equal those of the dense kernel on the pruned weight, compared on the GPU."""
