@@ -43,10 +43,10 @@ PEAK = {"op": ("mfma", 5.0e15, "TOP/s"),       # int8 dense MFMA
 # script summarised in TRAFFIC_SOURCE, each counter scaled by what it reads for the 1 GiB
 # --calibration-copy dispatch (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Counters cannot be read
 # from inside a timed run, so the figure is a recorded one: it is reported only for the default
-# workload (vit_h, batch 16, dense int8 linears) and only while the kernel's source file still
-# has the hash it had when the counters were taken (otherwise `traffic` is null).
+# workload (vit_h, batch 16, dense int8 linears) and only while the kernel family's source files
+# still have the hash they had when the counters were taken (otherwise `traffic` is null).
 TRAFFIC_SOURCE = "profiles/bench_vit_h_bs16_pmc_traffic.txt"
-TRAFFIC = {"gemm_i8_kernel": (1.0277e9, "gemm_i8.hip", "82d8a0dcda92f999")}
+TRAFFIC = {"gemm_i8_kernel": (1.0307e9, "gemm_i8.hip+gemm_i8_persist.hip+gemm_i8_shared.hpp", "2e4571a01cc60050")}
 
 
 def parse():
@@ -199,10 +199,16 @@ def library_yardsticks(batch, heads, hd, width):
     return res
 
 
-def source_sha16(name):
+def source_sha16(names):
+    """sha256 (first 16 hex digits) over the named kernel sources, in order ('a.hip+b.hip')"""
     import hashlib
-    path = ROOT / "segment-anything-fast_amd" / "csrc" / name
-    return hashlib.sha256(path.read_bytes()).hexdigest()[:16] if path.exists() else None
+    h = hashlib.sha256()
+    for name in names.split("+"):
+        path = ROOT / "segment-anything-fast_amd" / "csrc" / name
+        if not path.exists():
+            return None
+        h.update(path.read_bytes())
+    return h.hexdigest()[:16]
 
 
 def mfma_ceiling():
@@ -368,6 +374,38 @@ def gemm_variants(batch=16, width=1280):
             del xq, wq
         res["rows"][f"{name} {M}x{N}x{K}"] = row
         del y, resid
+    # the 2:4-sparse kernel's two forms on the MLP shapes (weights pruned to 2:4, Gaussian codes)
+    sparse_variants = [("one workgroup per tile", {"SAMFAST_SPARSE_PERSIST": 0}),
+                       ("resident workgroups", {"SAMFAST_SPARSE_PERSIST": 2})]
+    for name, N, K, epi in shapes[2:]:
+        w = (torch.randn((N, K), device=dev, generator=g) * 28).round().clamp(-127, 127)
+        w4 = w.view(N, K // 4, 4)
+        keep = torch.zeros_like(w4, dtype=torch.bool).scatter_(-1, w4.abs().topk(2, dim=-1).indices, True)
+        wc, widx = ops.prune24_pack((w4 * keep).view(N, K).to(torch.int8))
+        sx = torch.full((M,), 0.01, device=dev)
+        sw = torch.full((N,), 0.001, device=dev)
+        bias = torch.zeros((N,), device=dev)
+        y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        resid = torch.randn((M, N), device=dev, generator=g).to(torch.bfloat16) if epi == _lib.EPILOGUE_RESIDUAL else None
+        xq = (torch.randn((K // 64, M, 64), device=dev, generator=g) * 28).round().clamp(-127, 127).to(torch.int8)
+        run = lambda: ops.gemm_i8_sparse24_fused(xq, sx, wc, widx, sw, bias, epi, residual=resid, out=y,
+                                                 layout=_lib.LAYOUT_KB64)
+        row = {}
+        for label, knobs in sparse_variants:
+            with _lib.knobs(**knobs):
+                for _ in range(3):
+                    run()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(10):
+                    run()
+                e1.record()
+                torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 100.0
+            row[label] = {"gaussian": {"us": round(us, 1), "TOP/s executed": round(1.0 * M * N * K / us / 1e6, 1)}}
+        res["rows"][f"2:4 {name} {M}x{N}x{K}"] = row
+        del y, resid, xq, wc, widx
     torch.cuda.empty_cache()
     return res
 
