@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_persist_kernel(SparseArgs
   const int nt = (int)((last - first + per_x - 1u) / per_x);
 
   auto tile_origin = [&](unsigned int pid, int& x0, int& w0) __attribute__((always_inline)) {
-    constexpr unsigned int GROUP_X = 8;  // 1024 X rows per group: their panels stay in the XCD's L2
+    const unsigned int GROUP_X = (unsigned int)a.group_x;  // X panels per scheduling group
     const unsigned int per_group = GROUP_X * a.tiles_w;
     const unsigned int first_x = (pid / per_group) * GROUP_X;
     const unsigned int gsz = min((unsigned int)a.tiles_x - first_x, GROUP_X);

@@ -233,10 +233,10 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_kernel(SparseArgs a) {
   const unsigned int total = (unsigned int)a.tiles_x * (unsigned int)a.tiles_w;
   const unsigned int pid = xcd_contiguous_id(blockIdx.x, total);
   if (pid >= total) return;  // uniform over the workgroup
-  constexpr int GROUP_X = 8;  // 1024 X rows per group: their panels stay in the XCD's L2
+  const unsigned int GROUP_X = (unsigned int)a.group_x;  // X panels per scheduling group
   const unsigned int per_group = GROUP_X * a.tiles_w;
   const unsigned int first_x = (pid / per_group) * GROUP_X;
-  const unsigned int gsz = min((unsigned int)a.tiles_x - first_x, (unsigned int)GROUP_X);
+  const unsigned int gsz = min((unsigned int)a.tiles_x - first_x, GROUP_X);
   const unsigned int in_group = pid % per_group;
   const int x0 = (int)(first_x + in_group % gsz) * SBX;
   const int w0 = (int)(in_group / gsz) * SBW;
@@ -492,6 +492,10 @@ static int sparse_common(int epi, const int8_t* xq, const float* sx, const int8_
   a.ld_res = ld_res;
   a.tiles_x = (int)((M + SBX - 1) / SBX);
   a.tiles_w = (N + SBW - 1) / SBW;
+  // few column tiles (lin2: 5): the column tiles of one X panel run next to each other, the panel is
+  // fetched through the fabric once (2.0 instead of 3.6 GB per launch at 131072 x 1280 x 5120, -2 %);
+  // many column tiles (lin1: 20): groups of 8 X panels (1024 rows) whose panels stay in the XCD's L2
+  a.group_x = a.tiles_w <= 6 ? 1 : 8;
   const int64_t total = (int64_t)a.tiles_x * a.tiles_w;
   SF_REQUIRE(total < (1ll << 30), "gemm_i8_sparse24: too many tiles");
   if (gemm_i8_sp24_persist_covers(epi, a)) return gemm_i8_sp24_persist_launch(epi, a, stream);

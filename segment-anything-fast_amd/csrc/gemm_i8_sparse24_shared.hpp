@@ -29,6 +29,7 @@ struct SparseArgs {
   int64_t ldo;
   int M, N, K;
   int tiles_x, tiles_w;
+  int group_x;       // X panels (128 rows) per scheduling group
   int x_row_pitch;   // bytes between consecutive X rows: K (row-major) or 64 (K-block major)
   int64_t x_kstep;   // bytes between consecutive 64-byte k tiles of X: 64, or M * 64
   const unsigned short* residual;
