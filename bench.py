@@ -338,7 +338,8 @@ def gemm_variants(batch=16, width=1280):
     variants = [("three_workgroups_per_cu", {"SAMFAST_GEMM_PERSIST": 0}),
                 ("two_workgroups_per_cu", {"SAMFAST_GEMM_PERSIST": 0, "SAMFAST_GEMM_WG3": 0}),
                 ("persistent, all workgroups start together", {"SAMFAST_GEMM_PERSIST": 2, "SAMFAST_GEMM_PERSIST_SKEW": 0}),
-                ("persistent, every second workgroup starts a tile late", {"SAMFAST_GEMM_PERSIST": 2})]
+                ("persistent, every second workgroup starts a tile late", {"SAMFAST_GEMM_PERSIST": 2}),
+                ("persistent, skewed, no wave priorities", {"SAMFAST_GEMM_PERSIST": 2, "SAMFAST_GEMM_PERSIST_PRIO": 0})]
     shapes = [("qkv", 3 * width, width, _lib.EPILOGUE_NONE), ("proj", width, width, _lib.EPILOGUE_RESIDUAL),
               ("lin1", 4 * width, width, _lib.EPILOGUE_GELU), ("lin2", width, 4 * width, _lib.EPILOGUE_RESIDUAL)]
     res = {"what": f"gemm_i8 at M={M}, us per launch (10 back to back) and TOP/s, per variant knob, on "

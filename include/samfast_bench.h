@@ -16,7 +16,8 @@ extern "C" {
 /*
  * Kernel variants are chosen by knobs, each named like the environment variable that gives its
  * initial value (read once per process): SAMFAST_GEMM_TM, SAMFAST_GEMM_WG3, SAMFAST_GEMM_TILE,
- * SAMFAST_GEMM_SMALL_BELOW, SAMFAST_GEMM_PERSIST, SAMFAST_GEMM_PERSIST_SKEW, SAMFAST_GEMM_SPLITK,
+ * SAMFAST_GEMM_SMALL_BELOW, SAMFAST_GEMM_PERSIST, SAMFAST_GEMM_PERSIST_SKEW, SAMFAST_GEMM_PERSIST_PRIO,
+ * SAMFAST_GEMM_SPLITK,
  * SAMFAST_ATTN_WAVES, SAMFAST_ATTN_WINDOW_ROWS, SAMFAST_SPARSE_PERSIST.  This
  * call sets one (`unset` != 0: back to "not given", `value` ignored).  Every variant of a kernel
  * returns the same bits; the knobs only move time.  Returns SAMFAST_E_INVALID for an unknown name.

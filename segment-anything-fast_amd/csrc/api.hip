@@ -30,7 +30,7 @@ int check_launch(const char* what) {
 
 static const char* const kKnobNames[KNOB_COUNT] = {
     "SAMFAST_GEMM_TM",      "SAMFAST_GEMM_WG3",    "SAMFAST_GEMM_TILE", "SAMFAST_GEMM_SMALL_BELOW",
-    "SAMFAST_GEMM_PERSIST", "SAMFAST_GEMM_PERSIST_SKEW", "SAMFAST_GEMM_SPLITK", "SAMFAST_ATTN_WAVES", "SAMFAST_ATTN_WINDOW_ROWS",
+    "SAMFAST_GEMM_PERSIST", "SAMFAST_GEMM_PERSIST_SKEW", "SAMFAST_GEMM_PERSIST_PRIO", "SAMFAST_GEMM_SPLITK", "SAMFAST_ATTN_WAVES", "SAMFAST_ATTN_WINDOW_ROWS",
     "SAMFAST_SPARSE_PERSIST"};
 static int g_knobs[KNOB_COUNT];
 static pthread_once_t g_knobs_once = PTHREAD_ONCE_INIT;

@@ -984,6 +984,7 @@ static int gemm_common(int epi, const int8_t* xq, const float* sx, const int8_t*
   // (an output the quantiser tail reads back right away is not streamed past the caches)
   a.stream_out = !tail && (epi == EPI_SCALE_BIAS_BF16 || epi == EPI_GELU_BF16) && M * (int64_t)N * 2 >= (256ll << 20);
   a.skew = 0;
+  a.prio = 0;
   a.tile_counters = nullptr; a.yq = nullptr; a.sy = nullptr; a.ln_gamma = a.ln_beta = nullptr;
   a.ln_eps = 0.f; a.yq_kb64 = 0;
   if (tail) {

@@ -57,7 +57,7 @@ struct PersistIter {
   static constexpr int S0 = S0_, NSTORE = NSTORE_, D = D_, THRESH = THRESH_;
 };
 
-template <int EPI, int DI, int IMM, bool NT>
+template <int EPI, int DI, int IMM, bool NT, bool PRIO = true>
 __global__ __launch_bounds__(256, PERSIST_MIN_WG) void gemm_i8_persist_kernel(GemmArgs a) {
   static_assert(EPI == EPI_SCALE_BIAS_BF16 || EPI == EPI_GELU_BF16 || EPI == EPI_RESIDUAL_BF16, "epilogues built");
   constexpr bool RES = EPI == EPI_RESIDUAL_BF16;
@@ -279,6 +279,7 @@ __global__ __launch_bounds__(256, PERSIST_MIN_WG) void gemm_i8_persist_kernel(Ge
     constexpr bool ZERO = F::ZERO, CONV = F::CONV, SC = F::SC, ISSUE = F::ISSUE, NEXT = F::NEXT, RFIRST = F::RFIRST;
     constexpr int S0 = F::S0, NSTORE = F::NSTORE, THRESH = F::THRESH, D = F::D;
     if constexpr (CONV) {
+      if constexpr (PRIO) __builtin_amdgcn_s_setprio(0);
       // residual epilogue: the values requested in the last iteration have landed (its tile loads, the
       // youngest operations in flight, need not have)
       if constexpr (RES) __builtin_amdgcn_s_waitcnt(0x0F70 | PNLD);  // vmcnt <= PNLD, nothing else waited for
@@ -296,6 +297,7 @@ __global__ __launch_bounds__(256, PERSIST_MIN_WG) void gemm_i8_persist_kernel(Ge
       __builtin_amdgcn_sched_barrier(0);
       mma_zero_row(1, fa0, fb0);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (PRIO) __builtin_amdgcn_s_setprio(1);
       frags_at(st[0], 1, fa1, fb1);
     } else {
       frags_at(st[0], 1, fa1, fb1);
@@ -372,6 +374,11 @@ __global__ __launch_bounds__(256, PERSIST_MIN_WG) void gemm_i8_persist_kernel(Ge
   // plain iteration: tile loads only, one k tile in flight across the barrier
   using Plain = PersistIter<false, false, 0, 0, 0, false, false, true, true, PNLD>;
 
+  // A wavefront in its K loop runs at raised priority and drops to the base priority while it converts
+  // the previous tile's accumulators (PRIO): when its SIMD partner - the other resident workgroup's
+  // wavefront - is in its loop at that time, the partner's matrix instructions issue as soon as they
+  // are ready and the conversion's vector work fills the slots between them (lin1 + GELU -3 %).
+  //
   // Two resident workgroups that start in the same cycle run the same code on the same CU and tend
   // to stay in step: both in their LDS reads, both at their barriers, both converting.  The
   // workgroup whose first wavefront sits in an odd wave slot of its SIMD starts a.skew * 64 cycles late.
@@ -386,6 +393,7 @@ __global__ __launch_bounds__(256, PERSIST_MIN_WG) void gemm_i8_persist_kernel(Ge
       for (int i = 0; i < a.skew; ++i) __builtin_amdgcn_s_sleep(1);
   }
 
+  if constexpr (PRIO) __builtin_amdgcn_s_setprio(1);
   // ---- prologue: the first tile's scales and first three k tiles --------------------------------
   const int nk = a.K / GBK;
   int m0, n0;
@@ -499,23 +507,26 @@ int gemm_i8_persist_launch(int epi, const GemmArgs& a0, hipStream_t stream) {
   GemmArgs a = a0;
   // start delay of every second workgroup: knob x 64 cycles per k tile of a tile's K loop
   a.skew = min(max(knob_or(KNOB_GEMM_PERSIST_SKEW, 22), 0) * (a.K / GBK), 1 << 16);
+  a.prio = knob_or(KNOB_GEMM_PERSIST_PRIO, 1) != 0;
   a.tiles_m = a.M / PBM;
   a.tiles_n = a.N / PBN;
   a.group_m = a.tiles_n <= 6 ? 1 : 1024 / PBM;
   const int64_t total = (int64_t)a.tiles_m * a.tiles_n;
   const unsigned int grid = (unsigned int)min((int64_t)persist_grid(), ((total + 7) / 8) * 8);
   const bool di16 = a.K / GBK >= 20;
-#define SF_PERSIST(E)                                                                                            \
+#define SF_PERSIST_P(E, P)                                                                                       \
   do {                                                                                                           \
-    if (di16 && a.stream_out) hipLaunchKernelGGL((gemm_i8_persist_kernel<E, 16, 16, true>), dim3(grid), dim3(256), 0, stream, a);  \
-    else if (di16) hipLaunchKernelGGL((gemm_i8_persist_kernel<E, 16, 16, false>), dim3(grid), dim3(256), 0, stream, a);           \
-    else if (a.stream_out) hipLaunchKernelGGL((gemm_i8_persist_kernel<E, 8, 16, true>), dim3(grid), dim3(256), 0, stream, a);     \
-    else hipLaunchKernelGGL((gemm_i8_persist_kernel<E, 8, 16, false>), dim3(grid), dim3(256), 0, stream, a);                      \
+    if (di16 && a.stream_out) hipLaunchKernelGGL((gemm_i8_persist_kernel<E, 16, 16, true, P>), dim3(grid), dim3(256), 0, stream, a);  \
+    else if (di16) hipLaunchKernelGGL((gemm_i8_persist_kernel<E, 16, 16, false, P>), dim3(grid), dim3(256), 0, stream, a);           \
+    else if (a.stream_out) hipLaunchKernelGGL((gemm_i8_persist_kernel<E, 8, 16, true, P>), dim3(grid), dim3(256), 0, stream, a);     \
+    else hipLaunchKernelGGL((gemm_i8_persist_kernel<E, 8, 16, false, P>), dim3(grid), dim3(256), 0, stream, a);                      \
   } while (0)
+#define SF_PERSIST(E) do { if (a.prio) SF_PERSIST_P(E, true); else SF_PERSIST_P(E, false); } while (0)
   if (epi == EPI_GELU_BF16) SF_PERSIST(EPI_GELU_BF16);
   else if (epi == EPI_RESIDUAL_BF16) SF_PERSIST(EPI_RESIDUAL_BF16);
   else SF_PERSIST(EPI_SCALE_BIAS_BF16);
 #undef SF_PERSIST
+#undef SF_PERSIST_P
   return check_launch("gemm_i8_persist_kernel");
 }
 

@@ -22,6 +22,7 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int group_m;     // row tiles per scheduling group
   int stream_out;  // outputs without residual that exceed the 256 MB last-level cache
+  int prio;        // persistent kernel: 1 = wavefronts in their K loop run at raised priority, converting ones at base priority
   int skew;        // persistent kernel: start delay of the workgroups in odd wave slots, units of 64 cycles
   int row_pitch;            // bytes between consecutive rows of X / W: K (row-major) or 64 (K-block major)
   int64_t x_kstep, w_kstep; // bytes between consecutive 64-byte k tiles: 64, or rows * 64

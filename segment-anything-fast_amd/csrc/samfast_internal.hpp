@@ -31,6 +31,7 @@ enum Knob {
   KNOB_GEMM_SMALL_BELOW,  // SAMFAST_GEMM_SMALL_BELOW: tile count below which the small tile is taken
   KNOB_GEMM_PERSIST,      // SAMFAST_GEMM_PERSIST: 0 off, 1 where it pays, 2 wherever it is built
   KNOB_GEMM_PERSIST_SKEW, // SAMFAST_GEMM_PERSIST_SKEW: start delay of every second resident workgroup, 64 cycles per k tile
+  KNOB_GEMM_PERSIST_PRIO, // SAMFAST_GEMM_PERSIST_PRIO: 0 = no wave priority changes in the persistent kernel
   KNOB_GEMM_SPLITK,       // SAMFAST_GEMM_SPLITK: 0 off, 1 where it pays (launches that leave the GPU half empty)
   KNOB_ATTN_WAVES,        // SAMFAST_ATTN_WAVES: 4 / 8 wavefronts per global-attention workgroup
   KNOB_ATTN_WINDOW_ROWS,  // SAMFAST_ATTN_WINDOW_ROWS: 1 = window keys as grid rows padded to 16 (attn_window_rows_kernel) where built
