@@ -48,6 +48,15 @@ def test_knobs_are_named_and_bounded_without_gpu():
     assert lib.samfast_bench_set_knob(b"SAMFAST_GEMM_PERSIST", 0, 1) == 0
     assert lib.samfast_bench_set_knob(b"SAMFAST_NO_SUCH_KNOB", 1, 0) == -1
     assert b"unknown knob" in lib.samfast_last_error()
+    # every knob the bench header and the internal enumeration name is known to the library, and they
+    # name the same set
+    import re
+    root = Path(__file__).resolve().parents[1]
+    documented = set(re.findall(r"SAMFAST_(?:GEMM|ATTN|SPARSE)_[A-Z0-9_]+", (root / "include" / "samfast_bench.h").read_text()))
+    internal = set(re.findall(r"// (SAMFAST_[A-Z0-9_]+):", (root / "segment-anything-fast_amd" / "csrc" / "samfast_internal.hpp").read_text()))
+    assert documented == internal and len(documented) >= 11, documented ^ internal
+    for name in sorted(documented):
+        assert lib.samfast_bench_set_knob(name.encode(), 0, 1) == 0, name
     buf = ctypes.create_string_buffer(65536)
     p = ctypes.addressof(buf)
     p += (-p) % 16
