@@ -46,7 +46,7 @@ PEAK = {"op": ("mfma", 5.0e15, "TOP/s"),       # int8 dense MFMA
 # workload (vit_h, batch 16, dense int8 linears) and only while the kernel family's source files
 # still have the hash they had when the counters were taken (otherwise `traffic` is null).
 TRAFFIC_SOURCE = "profiles/bench_vit_h_bs16_pmc_traffic.txt"
-TRAFFIC = {"gemm_i8_kernel": (1.0307e9, "gemm_i8.hip+gemm_i8_persist.hip+gemm_i8_shared.hpp", "2e4571a01cc60050")}
+TRAFFIC = {"gemm_i8_kernel": (1.0042e9, "gemm_i8.hip+gemm_i8_persist.hip+gemm_i8_shared.hpp", "bfc90be515ad881e")}
 
 
 def parse():
