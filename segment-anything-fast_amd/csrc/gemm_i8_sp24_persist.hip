@@ -333,6 +333,9 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_persist_kernel(SparseArgs
     if constexpr (SC) scales_issue(sc_x0, sc_w0, sc_buf);
     if constexpr (ISSUE) dma_issue(ld_kt, st[0]);
     if constexpr (CONV) {
+      // the K loop runs at raised wave priority, the conversion at base priority: the SIMD partner's
+      // matrix instructions issue as soon as they are ready (lin1 840 -> 798 us)
+      __builtin_amdgcn_s_setprio(0);
       // (the fences keep the zero-initialised matrix instructions of a token half behind the
       // conversion of that half: hoisted above it, old and new accumulators would be live together)
       __builtin_amdgcn_sched_barrier(0);
@@ -346,6 +349,7 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_persist_kernel(SparseArgs
       convert_piece(QC<3>{}, conv_sc, QC<0>{}, QC<4>{});
       mma_zero_half(1, fa[P], fi[P], fb[P]);
       __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(1);
       if constexpr (NEXT) frags_at(st[1], fa[1 - P], fi[1 - P], fb[1 - P]);
     } else {
       if constexpr (NEXT) frags_at(st[1], fa[1 - P], fi[1 - P], fb[1 - P]);
@@ -391,6 +395,7 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_sp24_persist_kernel(SparseArgs
   using Plain0 = SpStep<0, false, false, false, false, true, true, QNLD>;
   using Plain1 = SpStep<1, false, false, false, false, true, true, QNLD>;
 
+  __builtin_amdgcn_s_setprio(1);
   // ---- prologue: the first tile's scales and first three k tiles --------------------------------
   const int nk = a.K / SBK;  // even and >= 8 (checked by the host)
   int x0, w0;
@@ -468,8 +473,8 @@ static int sp_persist_grid() {
 
 bool gemm_i8_sp24_persist_covers(int epi, const SparseArgs& a) {
   // 0 (default): one workgroup per tile always - this form measures level with it (lin1 / lin2 of
-  // ViT-H at 131072 rows: 906 against 870-895 us, 649 against 653 us); 1: from two tiles per
-  // resident workgroup on; 2: wherever this form is built
+  // ViT-H at 131072 rows inside the encoder: 798 against 805 us, 608 against 591 us); 1: from two
+  // tiles per resident workgroup on; 2: wherever this form is built
   const int mode = knob_or(KNOB_SPARSE_PERSIST, 0);
   if (mode <= 0) return false;
   if (epi != SEPI_SCALE_BIAS && epi != SEPI_GELU && epi != SEPI_RESIDUAL) return false;
