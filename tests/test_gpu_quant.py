@@ -614,9 +614,12 @@ def test_gemm_persistent_form_agrees(M, N, K, epi):
     with _lib.knobs(SAMFAST_GEMM_PERSIST=2):
         got = run()
         again = run()
+    with _lib.knobs(SAMFAST_GEMM_PERSIST=2, SAMFAST_GEMM_PERSIST_PRIO=0, SAMFAST_GEMM_PERSIST_SKEW=0):
+        plain = run()  # no wave priorities, no start skew: the other instantiation of the same kernel
     torch.cuda.synchronize()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     assert torch.equal(again.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(plain.view(torch.int16), want.view(torch.int16))
     # the oracle on rows spread over the first, a middle and the last row tile
     rows = torch.cat([torch.arange(0, 3), torch.arange(M // 2 - 1, M // 2 + 2), torch.arange(M - 3, M)])
     xq_r, sx_r = orq.quantize_rows_absmax(x[rows])
